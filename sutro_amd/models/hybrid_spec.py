@@ -2,8 +2,8 @@
 mixer and feed-forward, so attention layers, recurrent layers and layers that
 run both side by side can be ordered freely.
 
-A spec is built from a checkpoint's ``config.json`` (see :func:`vodinex_spec`
-and :func:`ruludra_spec`)
+A spec is built from a checkpoint's ``config.json`` (see :func:`vodinex_spec`,
+:func:`ruludra_spec` and :func:`vukotar_spec`)
 or directly in code (tests, benchmarks). Nothing here fixes a size: widths,
 head counts, mask sizes, filter lengths and the order of layers all come from
 the config.
@@ -37,6 +37,9 @@ class AttnMixerSpec:
     qk_norm: bool = True
     bias: bool = True        # q/k/v/o projections carry biases
     out_gate: bool = True    # one sigmoid gate per head on the attention output
+    # a silent sink: a key of score 0 without a value takes part in the
+    # normalisation, p_j = exp(s_j) / (1 + sum_j exp(s_j))
+    sink: bool = False
 
 
 @dataclass(frozen=True)
@@ -122,11 +125,37 @@ MixerSpec = Union[AttnMixerSpec, DeltaMixerSpec, ParallelMixerSpec,
 
 
 @dataclass(frozen=True)
+class RoutedExpertsSpec:
+    """Mixture-of-experts feed-forward: `experts` small two-matrix
+    feed-forwards of inner width `ff`, of which a token uses `top`.
+
+    ``router``: "sigmoid" scores every expert by the sigmoid of its logit and
+    weights the chosen ones by score / (sum of chosen scores + 1e-20).
+    ``groups`` / ``keep``: the experts form `groups` equal runs of neighbours;
+    a run is worth the sum of its `group_rank` largest scores and only experts
+    of the `keep` best runs can be chosen (groups = keep = 1: no restriction).
+    ``act``: "relu2" = the square of relu between the two matrices."""
+
+    ff: int
+    experts: int
+    top: int
+    groups: int = 1
+    keep: int = 1
+    group_rank: int = 2
+    router: str = "sigmoid"
+    act: str = "relu2"
+
+
+@dataclass(frozen=True)
 class HybridLayerSpec:
     kind: str                # the config's layer type
     mixer: MixerSpec
-    ff: int = 0              # 0 = the layer has no feed-forward sublayer
+    ff: int = 0              # 0 = the layer has no (dense) feed-forward
     ff_kind: str = "dense"
+    moe: Optional[RoutedExpertsSpec] = None
+    # index of the layer whose parameters this layer uses (its cache is its
+    # own); None = the layer has parameters of its own
+    weights_of: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -148,6 +177,8 @@ class HybridSpec:
     bigram: Optional[Tuple[int, int, int]] = None
     pos_base: float = 0.0        # base of the additive sinusoid (0 = none)
     logit_scale: float = 1.0
+    embed_scale: float = 1.0     # multiplies the token row
+    logit_softcap: float = 0.0   # c * tanh(logits / c); 0 = none
     # behavior flags shared with ModelSpec
     reasoning: bool = False
     embedding: bool = False
@@ -176,6 +207,8 @@ class HybridSpec:
 
         if self.arch == "ruludra":
             return self._sandwich_param_count()
+        if self.arch == "vukotar":
+            return self._parallel_param_count(active=False)
         for layer in self.layers:
             m = layer.mixer
             if isinstance(m, ParallelMixerSpec):
@@ -214,7 +247,28 @@ class HybridSpec:
                 n += 2 * h * layer.ff + 4 + 2 * h
         return n
 
+    def _parallel_param_count(self, active: bool) -> int:
+        """Tied embedding, Dynamic-Tanh norms, layer scales; layers that
+        borrow another layer's parameters add none. `active`: count only the
+        experts a token uses."""
+        h = self.hidden_size
+        n = self.vocab_size * h + 2 * h + 1
+        for layer in self.layers:
+            if layer.weights_of is not None and not active:
+                continue
+            m = layer.mixer
+            n += 2 * h + 1 + h
+            n += h * (m.heads * m.dim + m.kv_heads * (m.dim + m.vdim))
+            n += m.heads * m.vdim * h
+            if layer.moe:
+                e = layer.moe
+                n += h + e.experts * h
+                n += (e.top if active else e.experts) * 2 * h * e.ff
+        return n
+
     def active_param_count(self) -> int:
+        if self.arch == "vukotar":
+            return self._parallel_param_count(active=True)
         return self.param_count()
 
 
@@ -350,3 +404,71 @@ def ruludra_spec(config: dict, name: str = "ruludra",
         bigram=(int(big["buckets"]), int(big["mul_prev"]),
                 int(big["mul_cur"])) if big else None,
         pos_base=10000.0, logit_scale=float(config.get("logit_scale", 1.0)))
+
+
+def vukotar_spec(config: dict, name: str = "vukotar",
+                 checkpoint_dir: Optional[str] = None,
+                 tensor_shapes: Optional[dict] = None) -> HybridSpec:
+    """Build the spec of a Vukotar checkpoint from its ``config.json``: a
+    list of parallel layers (one Dynamic-Tanh norm feeding a sink-softmax
+    attention and a routed-experts feed-forward, each under a layer scale),
+    layers that borrow an earlier or later layer's tensors (``weights_of``),
+    scaled token embedding + sinusoid, tied and soft-capped logits."""
+    raw = config["layers"]
+
+    def owner(i: int) -> int:
+        seen = set()
+        while raw[i].get("weights_of") is not None:
+            if i in seen:
+                raise ValueError(f"layer {i}: weights_of runs in a circle")
+            seen.add(i)
+            i = int(raw[i]["weights_of"])
+            if not 0 <= i < len(raw):
+                raise ValueError("weights_of names no layer")
+        return i
+
+    layers = []
+    for i, lc in enumerate(raw):
+        kind = lc["type"]
+        if kind != "attention":
+            raise ValueError(f"unknown layer type {kind!r} in layer {i}")
+        m = lc["mixer"]
+        mixer = AttnMixerSpec(
+            heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+            dim=int(m["dim"]), vdim=int(m["vdim"]), scale=float(m["scale"]),
+            qk_norm=False, bias=False, out_gate=False, sink=True)
+        mlp = lc.get("mlp")
+        moe = None
+        if mlp is not None:
+            if mlp.get("kind") != "moe":
+                raise ValueError(f"unknown feed-forward kind {mlp.get('kind')!r}")
+            r = mlp["router"]
+            g = r.get("groups") or {"count": 1, "keep": 1}
+            moe = RoutedExpertsSpec(
+                ff=int(mlp["expert"]["ff"]), experts=int(r["experts"]),
+                top=int(r["top"]), groups=int(g["count"]), keep=int(g["keep"]))
+            if moe.experts % moe.groups or not 1 <= moe.keep <= moe.groups:
+                raise ValueError(f"layer {i}: experts must split into equal "
+                                 f"groups, of which 1..groups are kept")
+            if moe.top > moe.keep * (moe.experts // moe.groups):
+                raise ValueError(f"layer {i}: the kept groups hold fewer "
+                                 f"experts than a token uses")
+        own = owner(i)
+        layers.append(HybridLayerSpec(kind=kind, mixer=mixer, moe=moe,
+                                      weights_of=None if own == i else own))
+    for i, layer in enumerate(layers):
+        if layer.weights_of is not None:
+            src = layers[layer.weights_of]
+            if (src.mixer, src.moe) != (layer.mixer, layer.moe):
+                raise ValueError(f"layer {i} borrows the tensors of layer "
+                                 f"{layer.weights_of} but differs in shape")
+    return HybridSpec(
+        name=name, arch="vukotar", hidden_size=int(config["width"]),
+        vocab_size=int(config["vocab"]), layers=tuple(layers),
+        norm_eps=float(config["norm"]["eps"]),
+        max_context=int(config.get("max_context", 1 << 20)),
+        checkpoint_dir=checkpoint_dir, pos_base=10000.0,
+        embed_scale=float(config["embedding"]["scale"]),
+        logit_softcap=float(config.get("logit_softcap", 0.0) or 0.0),
+        tie_embeddings=True,
+        num_experts=max((l.moe.experts if l.moe else 0) for l in layers))

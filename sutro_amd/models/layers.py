@@ -19,7 +19,8 @@ from ..engine.batch import ForwardBatch
 from ..engine.kv_cache import PagedKVCache
 from ..ops import hybrid as hops
 from .hybrid_spec import (AttnMixerSpec, DeltaMixerSpec, LatentAttnMixerSpec,
-                          MLSTMMixerSpec, TiedAttnMixerSpec)
+                          MLSTMMixerSpec, RoutedExpertsSpec,
+                          TiedAttnMixerSpec)
 
 _ALIGN = 8  # section starts are multiples of 8 columns (16 B in bf16)
 
@@ -71,9 +72,12 @@ class SectionedLinear(nn.Module):
 class LocalAttention(nn.Module):
     """Grouped-query softmax attention under a chunk and/or window mask, with
     per-head q/k RMS norm, rotation of a prefix of each head, split key and
-    value sizes and a per-head sigmoid output gate. Owns no projection: it
-    works on sections of the sublayer's merged projection and writes its
-    gated heads into a slice of the merged output-projection input."""
+    value sizes, a per-head sigmoid output gate and an optional silent sink
+    in the softmax (each part can be switched off by the spec). Owns no
+    projection: it works on sections of the sublayer's merged projection and
+    writes its gated heads into a slice of the merged output-projection input.
+    `cache_idx` in forward names the layer whose pages are used when several
+    layers share this module's parameters."""
 
     def __init__(self, spec: AttnMixerSpec, eps: float, layer_idx: int):
         super().__init__()
@@ -107,11 +111,22 @@ class LocalAttention(nn.Module):
     def kv_shape(self):
         return (self.spec.kv_heads, self.spec.dim, self.spec.vdim)
 
+    def state_shape(self):
+        return None
+
+    def section_names(self, tag: str, ck: str):
+        n = {tag + "q": ck + ".q", tag + "k": ck + ".k", tag + "v": ck + ".v"}
+        if self.spec.out_gate:
+            n[tag + "g"] = ck + ".g"
+        return n
+
     def forward(self, proj: torch.Tensor, off: Dict[str, int], tag: str,
                 fb: ForwardBatch, kv: PagedKVCache, out: torch.Tensor,
-                out_off: int, out_scale: float) -> None:
+                out_off: int, out_scale: float,
+                cache_idx: Optional[int] = None) -> None:
         s = self.spec
-        kc, vc = kv.k_cache[self.layer_idx], kv.v_cache[self.layer_idx]
+        ci = self.layer_idx if cache_idx is None else cache_idx
+        kc, vc = kv.k_cache[ci], kv.v_cache[ci]
         cos_sin = None
         if proj.is_cuda:
             # one cos/sin table per step and kind of rotation, shared by layers
@@ -132,7 +147,7 @@ class LocalAttention(nn.Module):
             s.scale, s.chunk, s.window, proj,
             off[tag + "g"] if s.out_gate else -1, out, out_off, out_scale,
             token_seq=fb.token_seq, tile_seq=fb.tile_seq, tile_q0=fb.tile_q0,
-            prefill_rows=fb.prefill_token_count)
+            prefill_rows=fb.prefill_token_count, sink=s.sink)
 
 
 class GatedDeltaRule(nn.Module):
@@ -437,3 +452,56 @@ class MLSTM(nn.Module):
             fb.state_slots, fb.query_start_locs, fb.seq_lens)
         hops.mlstm_out(o, em, self.norm_w, proj, off[tag + "g"], self.eps,
                        out, out_off)
+
+
+class RoutedExperts(nn.Module):
+    """Mixture-of-experts feed-forward: a sigmoid router (fp32 logits) with
+    group-limited choice, and per expert `down act(up h)` without biases. The
+    chosen (token, expert) pairs are laid out in per-expert segments, the two
+    expert GEMMs run over the segments, and the caller folds the weighted sum
+    of a token's rows into its residual kernel: forward returns
+    (rows [padded rows, W], padpos [T, top], weights [T, top]).
+
+    Parameters are stacked [E, N, K] (each expert a torch-Linear matrix), the
+    layout the matrix-core expert GEMM reads."""
+
+    def __init__(self, spec: RoutedExpertsSpec, width: int,
+                 dtype: torch.dtype):
+        super().__init__()
+        if spec.router != "sigmoid" or spec.act != "relu2":
+            raise ValueError("RoutedExperts: unknown router or activation")
+        self.spec = spec
+        self.width = width
+        E, ff = spec.experts, spec.ff
+        self.router = nn.Parameter(torch.zeros(E, width, dtype=torch.float32))
+        self.up = nn.Parameter(torch.zeros(E, ff, width, dtype=dtype))
+        self.down = nn.Parameter(torch.zeros(E, width, ff, dtype=dtype))
+
+    def param_targets(self, prefix: str, ck: str):
+        s = self.spec
+        t = {ck + ".router": (prefix + "router", 0, 0, s.experts, 1.0)}
+        for e in range(s.experts):
+            t[f"{ck}.e{e}.up"] = (prefix + "up", 0, e, 1, 1.0)
+            t[f"{ck}.e{e}.down"] = (prefix + "down", 0, e, 1, 1.0)
+        return t
+
+    def route(self, h: torch.Tensor):
+        s = self.spec
+        logits = F.linear(h.float(), self.router)
+        return hops.moe_route(logits, s.top, s.groups, s.keep, s.group_rank)
+
+    def forward(self, h: torch.Tensor):
+        s = self.spec
+        T = h.shape[0]
+        idx, wts = self.route(h)
+        bm = hops.expert_gemm_tile(h, self.up, T * s.top)
+        row_tok, tile_off, counts, padpos = hops.moe_dispatch(idx, s.experts,
+                                                              bm)
+        n = row_tok.shape[0]
+        act = torch.empty((n, s.ff), dtype=h.dtype, device=h.device)
+        hops.expert_gemm(act, h, self.up, row_tok, tile_off, counts,
+                         hops.ACT_RELU2, bm)
+        rows = torch.empty((n, self.width), dtype=h.dtype, device=h.device)
+        hops.expert_gemm(rows, act, self.down, None, tile_off, counts,
+                         hops.ACT_NONE, bm)
+        return rows, padpos, wts

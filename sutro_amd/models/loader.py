@@ -85,6 +85,10 @@ def _load_by_targets(model: torch.nn.Module, path: str, strict: bool) -> int:
                 p.copy_(src.reshape(()).to(p.dtype))
             else:
                 dst = p.narrow(dim, start, length)
+                if length == 1 and dst.dim() == src.dim() + 1:
+                    # a tensor one axis short fills one index of that axis
+                    # (stacked per-expert matrices)
+                    dst = dst.squeeze(dim)
                 if tuple(dst.shape) != tuple(src.shape):
                     raise ValueError(
                         f"shape mismatch for {name}: checkpoint "

@@ -3,7 +3,9 @@ residuals, tanh-GELU gating, local (chunked / windowed) paged attention with
 split key/value sizes, partial rotation and an optional distance bias, the
 gated delta rule; hashed-bigram + sinusoid embedding, weighted norms around a
 sublayer with depth-weighted sums of all layer results, PolyNorm, tied-value
-attention prep, latent norms and gates, and the mLSTM.
+attention prep, latent norms and gates, the mLSTM; Dynamic-Tanh norms fused
+with layer-scaled parallel residuals, and routed experts (sigmoid router with
+group-limited choice, dispatch into per-expert segments, expert GEMMs).
 
 GPU tensors run the HIP kernels of the `sutro_amd._C_mix` extension
 (csrc/mix_*.hip), templated on the activation type: bf16 when the engine
@@ -105,13 +107,15 @@ def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
                     query_start_locs, scale: float, chunk: int, window: int,
                     proj, gate_off: int, out, out_off: int, out_scale: float,
                     token_seq=None, tile_seq=None, tile_q0=None,
-                    prefill_rows: int = 0, bias_r1=None, bias_r2=None):
+                    prefill_rows: int = 0, bias_r1=None, bias_r2=None,
+                    sink: bool = False):
     """`tile_seq`/`tile_q0` (int32, 32 query rows a tile) cover the first
     `prefill_rows` rows: on the GPU in bf16 those rows run on the MFMA kernel
     when page size and head sizes allow it; the remaining (single-token) rows
     and all other cases run on the generic one-wave-per-row kernel.
     `bias_r1` / `bias_r2` (fp32 [H]): r1[h] * ln(1 + r2[h] * (i - j)) is taken
-    off the score of query i and key j."""
+    off the score of query i and key j. `sink`: a key of score 0 without a
+    value joins every row's normalisation (a one in the denominator)."""
     if q.is_cuda:
         if tile_seq is None or tile_seq.numel() == 0:
             tile_seq = tile_q0 = None
@@ -120,12 +124,12 @@ def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
                                block_tables, seq_lens, query_start_locs,
                                token_seq, scale, chunk, window, proj,
                                gate_off, out_scale, tile_seq, tile_q0,
-                               prefill_rows, bias_r1, bias_r2)
+                               prefill_rows, bias_r1, bias_r2, sink)
         return
     torch_ref.local_attention(q, k_cache, v_cache, block_tables, seq_lens,
                               query_start_locs, scale, chunk, window, proj,
                               gate_off, out, out_off, out_scale,
-                              bias_r1=bias_r1, bias_r2=bias_r2)
+                              bias_r1=bias_r1, bias_r2=bias_r2, sink=sink)
 
 
 def delta_prep(proj, q_off, k_off, v_off, b_off, a1_off, H, G, dk, dv,
@@ -188,19 +192,20 @@ sinusoid_inv_freq = torch_ref.sinusoid_inv_freq
 
 
 def token_embed(ids, prev_ids, positions, embed_w, bigram_w, buckets: int,
-                mul_prev: int, mul_cur: int, inv_freq, out=None):
-    """fp32 [T, W] sum of the token row, the hashed bigram row (row `buckets`
-    where prev_ids < 0) and the sinusoid of the position."""
+                mul_prev: int, mul_cur: int, inv_freq, out=None,
+                scale: float = 1.0):
+    """fp32 [T, W] sum of `scale` times the token row, the hashed bigram row
+    (row `buckets` where prev_ids < 0) and the sinusoid of the position."""
     if out is None:
         out = torch.empty((ids.shape[0], embed_w.shape[1]),
                           dtype=torch.float32, device=ids.device)
     if ids.is_cuda:
         _mix().token_embed(out, ids, prev_ids, positions, embed_w, bigram_w,
-                           buckets, mul_prev, mul_cur, inv_freq)
+                           buckets, mul_prev, mul_cur, inv_freq, scale)
     else:
         out.copy_(torch_ref.token_embed(ids, prev_ids, positions, embed_w,
                                         bigram_w, buckets, mul_prev, mul_cur,
-                                        inv_freq))
+                                        inv_freq, scale))
     return out
 
 
@@ -286,3 +291,85 @@ def mlstm_out(o, em, norm_w, proj, g_off: int, eps: float, out,
         _mix().mlstm_out(out, out_off, o, em, norm_w, proj, g_off, eps)
         return
     torch_ref.mlstm_out(o, em, norm_w, proj, g_off, eps, out, out_off)
+
+
+# ---- Dynamic-Tanh norm with layer-scaled parallel residuals, routed
+# ---- experts, logit soft cap ----
+
+ACT_NONE, ACT_SILU_GATE, ACT_RELU2 = 0, 1, 2
+
+
+def dyt_residual(x, y1=None, ls1=None, y2=None, ls2=None, rows=None,
+                 padpos=None, wts=None, norm=None, h_out=None) -> None:
+    """x (fp32 [T, W], in place) += ls1 * y1 + ls2 * y2; the second branch is
+    y2 [T, W] or, with `rows`, the weighted sum of expert results
+    sum_j wts[t, j] * rows[padpos[t, j]]. Then h_out = tanh(alpha * x) * w + b
+    for norm = (alpha, w, b). Every part is optional; one kernel."""
+    alpha, nw, nb = norm if norm is not None else (None, None, None)
+    if x.is_cuda:
+        _mix().dyt_residual(x, y1, ls1, y2, ls2, rows, padpos, wts, alpha, nw,
+                            nb, h_out)
+        return
+    torch_ref.dyt_residual(x, y1, ls1, y2, ls2, rows, padpos, wts, alpha, nw,
+                           nb, h_out if norm is not None else None)
+
+
+def moe_route(logits, top: int, groups: int, keep: int, group_rank: int = 2):
+    """Sigmoid router with group-limited choice over fp32 logits [T, E]:
+    (idx int32 [T, top], weights fp32 [T, top])."""
+    if logits.is_cuda:
+        T = logits.shape[0]
+        idx = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+        w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+        _mix().moe_route(idx, w, logits, groups, keep, group_rank)
+        return idx, w
+    return torch_ref.moe_route(logits, top, groups, keep, group_rank)
+
+
+def moe_dispatch(idx, experts: int, bm: int):
+    """Per-expert segments padded to `bm` rows for idx int32 [T, k]:
+    (row_tok int32 [T*k + experts*bm], tile_off int32 [experts+1], counts
+    int32 [experts], padpos int32 [T, k]). One kernel, no host round trip."""
+    if idx.is_cuda:
+        T, k = idx.shape
+        dev = idx.device
+        row_tok = torch.empty(T * k + experts * bm, dtype=torch.int32,
+                              device=dev)
+        tile_off = torch.empty(experts + 1, dtype=torch.int32, device=dev)
+        counts = torch.empty(experts, dtype=torch.int32, device=dev)
+        padpos = torch.empty((T, k), dtype=torch.int32, device=dev)
+        _mix().moe_dispatch(row_tok, tile_off, counts, padpos, idx, bm)
+        return row_tok, tile_off, counts, padpos
+    return torch_ref.moe_dispatch(idx, experts, bm)
+
+
+def expert_gemm_tile(a, w, n_rows: int) -> int:
+    """Segment padding (rows) the expert GEMM of these operands wants: the
+    matrix-core kernel takes bf16 with K and N multiples of 64 and pads to
+    128 rows when segments are long; everything else runs the plain kernel on
+    64-row tiles."""
+    E = w.shape[0]
+    if a.is_cuda and a.dtype == torch.bfloat16 and n_rows >= E * 256:
+        return 128
+    return 64
+
+
+def expert_gemm(out, a, w, row_tok, tile_off, counts, act: int, bm: int):
+    """out[r] = act(a[row_tok[r]] @ w[e(r)]^T) over padded per-expert
+    segments (row_tok None: a is already laid out in segments). w [E, N, K];
+    act: ACT_NONE or ACT_RELU2."""
+    if out.is_cuda:
+        _mix().expert_gemm(out, a, w, row_tok, tile_off, counts, act, bm)
+        return out
+    return torch_ref.grouped_gemm(out, a, w, row_tok, tile_off, counts,
+                                  out.shape[0] // bm, act, bm)
+
+
+def softcap(logits, cap: float):
+    """fp32 cap * tanh(logits / cap)."""
+    if logits.is_cuda:
+        out = torch.empty(logits.shape, dtype=torch.float32,
+                          device=logits.device)
+        _mix().softcap(out, logits.contiguous(), cap)
+        return out
+    return torch_ref.softcap(logits, cap)

@@ -143,10 +143,14 @@ def topk_softmax_router(
 def grouped_gemm(out, a, w, row_tok, tile_off, counts, max_tiles, gate_silu,
                  bm: int = 64):
     """Reference for csrc/grouped_gemm.hip: per-expert segments padded to the
-    bm tile; gate_silu fuses silu(gate)*up over the two N-halves of w.
+    bm tile; gate_silu (True or 1) fuses silu(gate)*up over the two N-halves
+    of w; gate_silu == 2 squares relu of the single product (rows are still
+    gathered through row_tok).
     Padding rows of `out` are left untouched (the kernel writes deterministic
     garbage there; consumers must ignore them either way)."""
     E, N, K = w.shape
+    relu2 = int(gate_silu) == 2
+    gate_silu = int(gate_silu) == 1
     n_cols = N // 2 if gate_silu else N
     for e in range(E):
         c = int(counts[e])
@@ -162,6 +166,9 @@ def grouped_gemm(out, a, w, row_tok, tile_off, counts, max_tiles, gate_silu,
             g = rows @ w[e, :n_cols].T.float()
             u = rows @ w[e, n_cols:].T.float()
             out[s0:s0 + c] = (torch.nn.functional.silu(g) * u).to(out.dtype)
+        elif relu2:
+            z = torch.relu(rows @ w[e].T.float())
+            out[s0:s0 + c] = (z * z).to(out.dtype)
         else:
             out[s0:s0 + c] = (rows @ w[e].T.float()).to(out.dtype)
     return out
@@ -250,14 +257,16 @@ def attn_prep(proj, q_off, k_off, v_off, H, G, dk, dv, q_norm_w, k_norm_w,
 
 def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
                     query_start_locs, scale, chunk, window, proj, gate_off,
-                    out, out_off, out_scale, bias_r1=None, bias_r2=None):
+                    out, out_off, out_scale, bias_r1=None, bias_r2=None,
+                    sink=False):
     """Softmax attention of each sequence's new tokens over its cached keys
     under a local mask: query at position i sees j <= i with
     j >= (i // chunk) * chunk (chunk > 0) and j > i - window (window > 0).
     Head h's result is multiplied by out_scale * sigmoid(proj[t, gate_off+h])
     (gate_off < 0: no gate) and written to out[t, out_off + h*dv : ...].
     With bias_r1 / bias_r2 (fp32 [H]) the score of query i and key j is
-    lowered by r1[h] * ln(1 + r2[h] * (i - j))."""
+    lowered by r1[h] * ln(1 + r2[h] * (i - j)). With `sink` a key of score 0
+    that carries no value joins the normalisation."""
     T, H, dk = q.shape
     G, bs, dv = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
     rep = H // G
@@ -288,7 +297,12 @@ def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
         if window > 0:
             hidden = hidden | (kpos <= qpos - window)
         scores.masked_fill_(hidden.unsqueeze(0), float("-inf"))
-        o = torch.einsum("hqk,hkd->hqd", torch.softmax(scores, dim=-1), vh)
+        if sink:
+            zero = torch.zeros(H, nq, 1, dtype=scores.dtype, device=q.device)
+            pr = torch.softmax(torch.cat([scores, zero], -1), dim=-1)[..., :L]
+        else:
+            pr = torch.softmax(scores, dim=-1)
+        o = torch.einsum("hqk,hkd->hqd", pr, vh)
         o = o.transpose(0, 1) * out_scale                      # [nq, H, dv]
         if gate_off >= 0:
             o = o * torch.sigmoid(proj[q0:q1, gate_off:gate_off + H].float()).unsqueeze(-1)
@@ -407,12 +421,14 @@ def sinusoid_inv_freq(width: int, base: float) -> torch.Tensor:
 
 
 def token_embed(ids, prev_ids, positions, embed_w, bigram_w, buckets: int,
-                mul_prev: int, mul_cur: int, inv_freq):
-    """fp32 [T, W]: embed[id] (+ bigram[(prev*mul_prev + id*mul_cur) mod
+                mul_prev: int, mul_cur: int, inv_freq, scale: float = 1.0):
+    """fp32 [T, W]: scale * embed[id] (+ bigram[(prev*mul_prev + id*mul_cur) mod
     buckets], row `buckets` where prev < 0) (+ the sinusoid of the position:
     column 2i = sin(p * inv_freq[i]), column 2i+1 = cos of the same fp32
     angle)."""
     x = embed_w[ids].float()
+    if scale != 1.0:
+        x = x * scale
     if bigram_w is not None:
         row = (prev_ids * mul_prev + ids * mul_cur) % buckets
         row = torch.where(prev_ids < 0, torch.full_like(row, buckets), row)
@@ -560,3 +576,91 @@ def mlstm_out(o, em, norm_w, proj, g_off: int, eps: float, out, out_off: int):
     h = _unit_rms(h, eps).reshape(T, H * dv) * norm_w.float()
     h = h * torch.sigmoid(proj[:, g_off:g_off + H * dv].float())
     out[:, out_off:out_off + H * dv] = h.to(out.dtype)
+
+
+# --------------------------------------------------------------------------
+# Parallel layers under one Dynamic-Tanh norm, layer scales, routed experts.
+# --------------------------------------------------------------------------
+
+
+def moe_combine_rows(rows, padpos, w):
+    """fp32 [T, W]: sum_j w[t, j] * rows[padpos[t, j]]."""
+    return (rows[padpos.long()].float() * w.unsqueeze(-1)).sum(dim=1)
+
+
+def dyt_residual(x, y1, ls1, y2, ls2, rows, padpos, wts, alpha, nw, nb,
+                 h_out):
+    """x (fp32, in place) += ls1 * y1 + ls2 * y2, where the second branch is
+    either y2 [T, W] or the weighted sum of expert rows
+    sum_j wts[t, j] * rows[padpos[t, j]] (both None: one branch; y1 None: no
+    update). Then, unless h_out is None, h_out = tanh(alpha * x) * nw + nb
+    (alpha a 0-d tensor) in h_out's type."""
+    if y1 is not None:
+        add = y1.float() * ls1
+        if y2 is not None:
+            add = add + y2.float() * ls2
+        elif rows is not None:
+            add = add + moe_combine_rows(rows, padpos, wts) * ls2
+        x.add_(add)
+    if h_out is not None:
+        h_out.copy_((torch.tanh(alpha * x) * nw + nb).to(h_out.dtype))
+
+
+def moe_route(logits, top: int, groups: int, keep: int, group_rank: int = 2):
+    """Sigmoid router with group-limited choice. logits fp32 [T, E]. Returns
+    (idx int32 [T, top], weights fp32 [T, top]): the `top` largest sigmoid
+    scores among the experts of the `keep` groups (equal runs of neighbours)
+    whose `group_rank` largest scores sum highest, each divided by the sum of
+    the chosen scores + 1e-20. Ties go to the lower index."""
+    T, E = logits.shape
+    s = torch.sigmoid(logits.float())
+    if groups > 1:
+        size = E // groups
+        per = s.view(T, groups, size)
+        worth = per.topk(min(group_rank, size), dim=-1).values.sum(-1)
+        # stable descending order: ties keep the lower group
+        order = torch.sort(worth, dim=-1, descending=True, stable=True).indices
+        allow = torch.zeros(T, groups, dtype=torch.bool, device=s.device)
+        allow.scatter_(1, order[:, :keep], True)
+        masked = torch.where(allow.unsqueeze(-1), per,
+                             torch.full_like(per, -1.0)).reshape(T, E)
+    else:
+        masked = s
+    idx = torch.sort(masked, dim=-1, descending=True,
+                     stable=True).indices[:, :top]
+    w = s.gather(1, idx)
+    w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    return idx.to(torch.int32), w
+
+
+def moe_dispatch(idx, experts: int, bm: int):
+    """Lay the (token, choice) pairs of idx [T, k] out in per-expert segments
+    padded to `bm` rows. Returns (row_tok int32 [T*k + experts*bm]: the token
+    of every padded row, -1 for padding; tile_off int32 [experts+1]: segment
+    starts in tiles; counts int32 [experts]; padpos int32 [T, k]: the padded
+    row of every pair)."""
+    T, k = idx.shape
+    dev = idx.device
+    flat = idx.reshape(-1).long()
+    order = torch.argsort(flat, stable=True)
+    counts = torch.bincount(flat, minlength=experts)
+    padded = (counts + bm - 1) // bm * bm
+    pad_off = torch.zeros(experts + 1, dtype=torch.long, device=dev)
+    pad_off[1:] = torch.cumsum(padded, 0)
+    first = torch.zeros(experts + 1, dtype=torch.long, device=dev)
+    first[1:] = torch.cumsum(counts, 0)
+    se = flat[order]
+    pos = torch.arange(T * k, device=dev) - first[se]
+    where = pad_off[se] + pos
+    row_tok = torch.full((T * k + experts * bm,), -1, dtype=torch.int32,
+                         device=dev)
+    row_tok[where] = (order // k).to(torch.int32)
+    padpos = torch.empty(T * k, dtype=torch.int32, device=dev)
+    padpos[order] = where.to(torch.int32)
+    return (row_tok, (pad_off // bm).to(torch.int32), counts.to(torch.int32),
+            padpos.view(T, k))
+
+
+def softcap(logits, cap: float):
+    """cap * tanh(logits / cap) in fp32."""
+    return cap * torch.tanh(logits.float() / cap)
