@@ -14,6 +14,8 @@
 //       rows [0,m), up rows [m,2m) of the expert's weight) and the SwiGLU
 //       is fused into the epilogue — the 2m-wide intermediate never exists.
 //   stage 2 (gate_silu=0): out[r, 0:h]   = act[r] @ Wd[e]^T
+//   ungated stage 1 (gate_silu=2): act[r, 0:m] = relu(x[tok[r]] @ Wu[e]^T)^2
+//       (one B stream; experts of the form down(relu(up x)^2))
 //
 // Weights are stored [E, N, K] K-contiguous (torch-Linear layout per
 // expert), so MFMA fragments are 8 consecutive bf16 along K for both
@@ -87,10 +89,11 @@ __device__ __forceinline__ const bf16x8* gg_frag(const u16* lds, int row,
   return (const bf16x8*)((const char*)lds + gswz(lb));
 }
 
-// GATE_SILU=1: B has two streams (gate/up at N-offset 0 and n_cols), output
-// n_cols wide with silu(g)*u. GATE_SILU=0: plain B, plain store.
+// MODE=1: rows gathered, B has two streams (gate/up at N-offset 0 and n_cols), output
+// n_cols wide with silu(g)*u. MODE=0: plain A, plain B, plain store.
+// MODE=2: rows gathered, one B stream, relu(x)^2 in the epilogue.
 // Waves arranged WROWS(M) x WCOLS(N); wave tile = (BM/WROWS) x (BN/WCOLS).
-template <int GATE_SILU, int BM, int BN, int WROWS, int WCOLS>
+template <int MODE, int BM, int BN, int WROWS, int WCOLS>
 __global__ __launch_bounds__(WROWS* WCOLS * 64) void grouped_gemm_kernel(
     u16* __restrict__ out,        // [rows_max, n_cols] bf16
     const u16* __restrict__ a,    // GATHER: [T, K]; else [rows_max, K]
@@ -99,6 +102,8 @@ __global__ __launch_bounds__(WROWS* WCOLS * 64) void grouped_gemm_kernel(
     const int* __restrict__ tile_off,   // [E+1] padded-offset / BM
     const int* __restrict__ counts,     // [E] live rows per expert
     int n_experts, int n_cols, long K) {
+  constexpr bool GATED = MODE == 1;   // silu(gate) * up over two B streams
+  constexpr bool GATHER = MODE != 0;  // A rows come through row_tok
   constexpr int WAVES = WROWS * WCOLS;
   constexpr int WM = BM / WROWS;
   constexpr int WN = BN / WCOLS;
@@ -123,34 +128,34 @@ __global__ __launch_bounds__(WROWS* WCOLS * 64) void grouped_gemm_kernel(
   const int wave = threadIdx.x >> 6;
   const int wm = wave / WCOLS, wn = wave % WCOLS;
 
-  __shared__ u16 smem[2][(BM + (GATE_SILU ? 2 : 1) * BN) * 64];
+  __shared__ u16 smem[2][(BM + (MODE == 1 ? 2 : 1) * BN) * 64];
   const int b_off = BM * 64;
   const int b2_off = (BM + BN) * 64;
 
   const long Kb = K * 2;
-  const u16* wa = w + (long)e * (GATE_SILU ? 2 : 1) * n_cols * K;
+  const u16* wa = w + (long)e * (GATED ? 2 : 1) * n_cols * K;
   const u16* wg = wa + (long)n0 * K;
   const u16* wu = wa + (long)(n_cols + n0) * K;       // up rows (stage 1)
-  const u16* aa = GATE_SILU ? a : a + (long)seg0 * K;
+  const u16* aa = GATHER ? a : a + (long)seg0 * K;
   const int* rt = row_tok ? row_tok + seg0 : nullptr;
 
-  f32x4 accg[MF][NF], accu[GATE_SILU ? MF : 1][GATE_SILU ? NF : 1];
+  f32x4 accg[MF][NF], accu[GATED ? MF : 1][GATED ? NF : 1];
 #pragma unroll
   for (int i = 0; i < MF; ++i)
 #pragma unroll
     for (int j = 0; j < NF; ++j) {
       accg[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (GATE_SILU) accu[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (GATED) accu[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
   // prologue
-  if (GATE_SILU)
+  if (GATHER)
     gg_stage<BM, WAVES, true>(smem[0], aa, Kb, rt, m0, rows_valid, wave, lane);
   else
     gg_stage<BM, WAVES, false>(smem[0], aa, Kb, nullptr, m0, BM, wave, lane);
   gg_stage<BN, WAVES, false>(smem[0] + b_off, wg, Kb, nullptr, 0, BN, wave,
                              lane);
-  if (GATE_SILU)
+  if (GATED)
     gg_stage<BN, WAVES, false>(smem[0] + b2_off, wu, Kb, nullptr, 0, BN, wave,
                                lane);
   __syncthreads();
@@ -163,7 +168,7 @@ __global__ __launch_bounds__(WROWS* WCOLS * 64) void grouped_gemm_kernel(
     u16* buT = smem[p] + b2_off;
     if (kt + 1 < KT) {
       const long ko = (long)(kt + 1) * 64;
-      if (GATE_SILU)
+      if (GATHER)
         gg_stage<BM, WAVES, true>(smem[p ^ 1], aa + ko, Kb, rt, m0,
                                   rows_valid, wave, lane);
       else
@@ -171,18 +176,18 @@ __global__ __launch_bounds__(WROWS* WCOLS * 64) void grouped_gemm_kernel(
                                    wave, lane);
       gg_stage<BN, WAVES, false>(smem[p ^ 1] + b_off, wg + ko, Kb, nullptr, 0,
                                  BN, wave, lane);
-      if (GATE_SILU)
+      if (GATED)
         gg_stage<BN, WAVES, false>(smem[p ^ 1] + b2_off, wu + ko, Kb, nullptr,
                                    0, BN, wave, lane);
     }
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       const int kk16 = kk * 4 + (lane >> 4);
-      bf16x8 bg[NF], bu[GATE_SILU ? NF : 1];
+      bf16x8 bg[NF], bu[GATED ? NF : 1];
 #pragma unroll
       for (int j = 0; j < NF; ++j) {
         bg[j] = *gg_frag(bgT, wn * WN + j * 16 + (lane & 15), kk16);
-        if (GATE_SILU)
+        if (GATED)
           bu[j] = *gg_frag(buT, wn * WN + j * 16 + (lane & 15), kk16);
       }
 #pragma unroll
@@ -192,7 +197,7 @@ __global__ __launch_bounds__(WROWS* WCOLS * 64) void grouped_gemm_kernel(
 #pragma unroll
         for (int j = 0; j < NF; ++j) {
           accg[i][j] = mfma16g(af, bg[j], accg[i][j]);
-          if (GATE_SILU) accu[i][j] = mfma16g(af, bu[j], accu[i][j]);
+          if (GATED) accu[i][j] = mfma16g(af, bu[j], accu[i][j]);
         }
       }
     }
@@ -213,9 +218,13 @@ __global__ __launch_bounds__(WROWS* WCOLS * 64) void grouped_gemm_kernel(
         const int grow = grow0 + r;
         const long o = (long)(seg0 + m0 + grow) * n_cols + gn;
         float v = accg[i][j][r];
-        if (GATE_SILU) {
+        if (GATED) {
           const float g = v;
           v = g / (1.0f + __expf(-g)) * accu[i][j][r];
+        }
+        if (MODE == 2) {
+          v = fmaxf(v, 0.f);
+          v *= v;
         }
         out[o] = f2bf(v);
       }
@@ -243,14 +252,17 @@ extern "C" void sutro_grouped_gemm(void* out, const void* a, const void* w,
   /* no hipGetLastError in this launcher: error-state queries are rejected
      while a stream is capturing (decode steps replay under hipGraphs) */
   if (bm == 128 && n_cols % 128 == 0) {
-    if (gate_silu) GG_LAUNCH(1, 128, 128, 2, 4)
+    if (gate_silu == 1) GG_LAUNCH(1, 128, 128, 2, 4)
+    else if (gate_silu == 2) GG_LAUNCH(2, 128, 128, 2, 4)
     else GG_LAUNCH(0, 128, 128, 2, 4)
   }
   if (bm == 128) {
-    if (gate_silu) GG_LAUNCH(1, 128, 64, 4, 2)
+    if (gate_silu == 1) GG_LAUNCH(1, 128, 64, 4, 2)
+    else if (gate_silu == 2) GG_LAUNCH(2, 128, 64, 4, 2)
     else GG_LAUNCH(0, 128, 64, 4, 2)
   }
-  if (gate_silu) GG_LAUNCH(1, 64, 64, 2, 2)
+  if (gate_silu == 1) GG_LAUNCH(1, 64, 64, 2, 2)
+  else if (gate_silu == 2) GG_LAUNCH(2, 64, 64, 2, 2)
   else GG_LAUNCH(0, 64, 64, 2, 2)
 #undef GG_LAUNCH
 }

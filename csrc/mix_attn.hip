@@ -216,8 +216,8 @@ __global__ void local_attention_kernel(
     const int* __restrict__ qlocs, const int* __restrict__ token_seq,
     float scale, int chunk, int window, const A* __restrict__ proj, long ld,
     int gate_off, float out_scale, const float* __restrict__ bias_r1,
-    const float* __restrict__ bias_r2, long t0, long T, int H, int G, int dk,
-    int dv, int page) {
+    const float* __restrict__ bias_r2, int sink, long t0, long T, int H, int G,
+    int dk, int dv, int page) {
   extern __shared__ float sm[];  // WPB * dk floats: the wave's query
   const int lane = threadIdx.x & (WAVE - 1);
   const int wid = threadIdx.x / WAVE;
@@ -242,7 +242,8 @@ __global__ void local_attention_kernel(
   const float r1 = bias_r1 ? bias_r1[h] : 0.f;
   const float r2 = bias_r1 ? bias_r2[h] : 0.f;
 
-  float m = -INFINITY, l = 0.f;
+  // a sink is a key of score 0 without a value that is always visible
+  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
   float acc[NV];
 #pragma unroll
   for (int c = 0; c < NV; ++c) acc[c] = 0.f;
@@ -317,8 +318,8 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(
     const int* __restrict__ qlocs, const int* __restrict__ token_seq,
     float scale, int chunk, int window, const A* __restrict__ proj, long ld,
     int gate_off, float out_scale, const float* __restrict__ bias_r1,
-    const float* __restrict__ bias_r2, long t0, int H, int G, int dk, int dv,
-    int page) {
+    const float* __restrict__ bias_r2, int sink, long t0, int H, int G, int dk,
+    int dv, int page) {
   typedef typename Vec16<A>::type vec_t;
   constexpr int EPL = 16 / sizeof(A);     // elements per lane
   constexpr int KPI = 64 / LPR;           // keys per load instruction
@@ -436,7 +437,9 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(
   float mx = comb[0];  // wave 0 always has a tile
 #pragma unroll
   for (int w = 1; w < WPB; ++w) mx = fmaxf(mx, comb[w * CS]);
-  float wgt[WPB], lsum = 0.f;
+  // a sink (score 0, no value) joins the normalisation here, once per row
+  if (sink) mx = fmaxf(mx, 0.f);
+  float wgt[WPB], lsum = sink ? expf(-mx) : 0.f;
 #pragma unroll
   for (int w = 0; w < WPB; ++w) {
     wgt[w] = expf(comb[w * CS] - mx);   // a wave without tiles: exp(-inf) = 0
@@ -502,8 +505,8 @@ static void launch_local_attention(
     const void* v_cache, const int* bt, int bt_stride, const int* seq_lens,
     const int* qlocs, const int* token_seq, float scale, int chunk,
     int window, const void* proj, long ld, int gate_off, float out_scale,
-    const float* bias_r1, const float* bias_r2, long t0, long T, int H, int G,
-    int dk, int dv, int page, hipStream_t s) {
+    const float* bias_r1, const float* bias_r2, int sink, long t0, long T,
+    int H, int G, int dk, int dv, int page, hipStream_t s) {
   const long units = T * H;
   const int grid = (int)((units + WPB - 1) / WPB);
   if (grid == 0) return;
@@ -519,8 +522,8 @@ static void launch_local_attention(
                      ldo, out_off, (const A*)q, (const A*)k_cache,            \
                      (const A*)v_cache, bt, bt_stride, seq_lens, qlocs,       \
                      token_seq, scale, chunk, window, (const A*)proj, ld,     \
-                     gate_off, out_scale, bias_r1, bias_r2, t0, H, G, dk, dv, \
-                     page)
+                     gate_off, out_scale, bias_r1, bias_r2, sink, t0, H, G,   \
+                     dk, dv, page)
       if (lpr == 2) LAUNCH_LR(2);
       else if (lpr == 4) LAUNCH_LR(4);
       else if (lpr == 8) LAUNCH_LR(8);
@@ -538,7 +541,7 @@ static void launch_local_attention(
                      (const A*)q, (const A*)k_cache, (const A*)v_cache, bt,  \
                      bt_stride, seq_lens, qlocs, token_seq, scale, chunk,    \
                      window, (const A*)proj, ld, gate_off, out_scale,        \
-                     bias_r1, bias_r2, t0, T, H, G, dk, dv, page)
+                     bias_r1, bias_r2, sink, t0, T, H, G, dk, dv, page)
   if (dv <= 64) LAUNCH_LA(1);
   else if (dv <= 128) LAUNCH_LA(2);
   else if (dv <= 256) LAUNCH_LA(4);
@@ -551,18 +554,18 @@ extern "C" void mix_local_attention(
     const void* v_cache, const int* bt, int bt_stride, const int* seq_lens,
     const int* qlocs, const int* token_seq, float scale, int chunk,
     int window, const void* proj, long ld, int gate_off, float out_scale,
-    const float* bias_r1, const float* bias_r2, long t0, long T, int H, int G,
-    int dk, int dv, int page, int f32, hipStream_t s) {
+    const float* bias_r1, const float* bias_r2, int sink, long t0, long T,
+    int H, int G, int dk, int dv, int page, int f32, hipStream_t s) {
   if (f32)
     launch_local_attention<float>(out, ldo, out_off, q, k_cache, v_cache, bt,
                                   bt_stride, seq_lens, qlocs, token_seq, scale,
                                   chunk, window, proj, ld, gate_off, out_scale,
-                                  bias_r1, bias_r2, t0, T, H, G, dk, dv, page,
-                                  s);
+                                  bias_r1, bias_r2, sink, t0, T, H, G, dk, dv,
+                                  page, s);
   else
     launch_local_attention<u16>(out, ldo, out_off, q, k_cache, v_cache, bt,
                                 bt_stride, seq_lens, qlocs, token_seq, scale,
                                 chunk, window, proj, ld, gate_off, out_scale,
-                                bias_r1, bias_r2, t0, T, H, G, dk, dv, page,
-                                s);
+                                bias_r1, bias_r2, sink, t0, T, H, G, dk, dv,
+                                page, s);
 }

@@ -52,8 +52,8 @@ local_attention_mfma_kernel(
     const int* __restrict__ qlocs, const int* __restrict__ tile_seq,
     const int* __restrict__ tile_q0, float scale, int chunk, int window,
     const u16* __restrict__ proj, long ld, int gate_off, float out_scale,
-    const float* __restrict__ bias_r1, const float* __restrict__ bias_r2, int H,
-    int Hk, int dk, int dv, int parts) {
+    const float* __restrict__ bias_r1, const float* __restrict__ bias_r2,
+    int sink, int H, int Hk, int dk, int dv, int parts) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int w = threadIdx.x / WAVE;
   const int G = blockDim.x / WAVE;        // query heads of this workgroup
@@ -100,7 +100,9 @@ local_attention_mfma_kernel(
   f32x16 acc[DVP / 32];
 #pragma unroll
   for (int b = 0; b < DVP / 32; ++b) acc[b] = (f32x16)(0.f);
-  float m_run = -1e30f, l_run = 0.f;
+  // a sink (a key of score 0 without a value) starts the running maximum at
+  // 0 and the running sum at its weight
+  float m_run = sink ? 0.f : -1e30f, l_run = sink ? 1.f : 0.f;
   // distance bias of this wave's head: r1 * ln(1 + r2 * (p - j))
   const float r1 = bias_r1 ? bias_r1[hq] : 0.f;
   const float r2 = bias_r1 ? bias_r2[hq] : 0.f;
@@ -225,7 +227,7 @@ extern "C" int mix_local_attention_mfma(
     const int* qlocs, const int* tile_seq, const int* tile_q0, int n_tiles,
     float scale, int chunk, int window, const void* proj, long ld,
     int gate_off, float out_scale, const float* bias_r1, const float* bias_r2,
-    int H, int Hk, int dk, int dv, int page, hipStream_t s) {
+    int sink, int H, int Hk, int dk, int dv, int page, hipStream_t s) {
   if (page != PG || dk % 8 || dv % 8 || dk > 256 || dv > 256 || H % Hk)
     return 0;
   const int DKP = dk <= 64 ? 64 : (dk <= 128 ? 128 : 256);
@@ -251,7 +253,7 @@ extern "C" int mix_local_attention_mfma(
                      (const u16*)v_cache, bt, bt_stride, seq_lens, qlocs,     \
                      tile_seq, tile_q0, scale, chunk, window,                 \
                      (const u16*)proj, ld, gate_off, out_scale, bias_r1,     \
-                     bias_r2, H, Hk, dk, dv, parts)
+                     bias_r2, sink, H, Hk, dk, dv, parts)
   if (DKP == 64) {
     if (DVP == 64) LAUNCH_M(64, 64);
     else if (DVP == 128) LAUNCH_M(64, 128);

@@ -49,17 +49,32 @@ void mix_attn_prep(void*, const void*, long, int, int, int, const float*,
 void mix_local_attention(void*, long, int, const void*, const void*,
                          const void*, const int*, int, const int*, const int*,
                          const int*, float, int, int, const void*, long, int,
-                         float, const float*, const float*, long, long, int,
-                         int, int, int, int, int, hipStream_t);
+                         float, const float*, const float*, int, long, long,
+                         int, int, int, int, int, int, hipStream_t);
 int mix_local_attention_mfma(void*, long, int, const void*, const void*,
                              const void*, const int*, int, const int*,
                              const int*, const int*, const int*, int, float,
                              int, int, const void*, long, int, float,
                              const float*, const float*, int, int, int, int,
-                             int, hipStream_t);
+                             int, int, hipStream_t);
 void mix_token_embed(float*, const long*, const long*, const long*,
                      const void*, const void*, long, long, long, const float*,
-                     long, int, int, hipStream_t);
+                     float, long, int, int, hipStream_t);
+void mix_dyt_residual(float*, const void*, const float*, const void*,
+                      const float*, const void*, const int*, const float*, int,
+                      const float*, const float*, const float*, void*, long,
+                      int, int, hipStream_t);
+void mix_moe_route(int*, float*, const float*, long, int, int, int, int, int,
+                   hipStream_t);
+void mix_moe_dispatch(int*, int*, int*, int*, const int*, long, int, int, int,
+                      long, hipStream_t);
+void mix_expert_gemm_plain(void*, const void*, const void*, const int*,
+                           const int*, const int*, int, int, int, int, long,
+                           int, int, hipStream_t);
+void mix_softcap(float*, const void*, float, long, int, hipStream_t);
+void sutro_grouped_gemm(void*, const void*, const void*, const int*,
+                        const int*, const int*, int, int, int, long, int,
+                        int, hipStream_t);
 void mix_weighted_rmsnorm(void*, const float*, const float*, float, long, int,
                           int, hipStream_t);
 void mix_norm_residual(const float*, const void*, const float*, float, float*,
@@ -195,7 +210,7 @@ void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
                      c10::optional<torch::Tensor> tile_seq,
                      c10::optional<torch::Tensor> tile_q0,
                      long prefill_rows, c10::optional<torch::Tensor> bias_r1,
-                     c10::optional<torch::Tensor> bias_r2) {
+                     c10::optional<torch::Tensor> bias_r2, bool sink) {
   CHECK_GPU(q); CHECK_CONTIG(q); CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
   CHECK_I32(bt); CHECK_I32(seq_lens); CHECK_I32(qlocs); CHECK_I32(token_seq);
   CHECK_CONTIG(bt);
@@ -240,7 +255,8 @@ void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
             tile_seq->data_ptr<int>(), tile_q0->data_ptr<int>(),
             (int)tile_seq->numel(), (float)scale, (int)chunk, (int)window,
             proj.data_ptr(), proj.stride(0), (int)gate_off, (float)out_scale,
-            r1, r2, (int)H, (int)G, (int)dk, (int)dv, (int)page, cur_stream()))
+            r1, r2, sink ? 1 : 0, (int)H, (int)G, (int)dk, (int)dv, (int)page,
+            cur_stream()))
       t0 = prefill_rows;
   }
   if (t0 < T)
@@ -250,8 +266,8 @@ void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
                         seq_lens.data_ptr<int>(), qlocs.data_ptr<int>(),
                         token_seq.data_ptr<int>(), (float)scale, (int)chunk,
                         (int)window, proj.data_ptr(), proj.stride(0),
-                        (int)gate_off, (float)out_scale, r1, r2, t0, T - t0,
-                        (int)H,
+                        (int)gate_off, (float)out_scale, r1, r2, sink ? 1 : 0,
+                        t0, T - t0, (int)H,
                         (int)G, (int)dk, (int)dv, (int)page, act_kind(q),
                         cur_stream());
 }
@@ -369,7 +385,7 @@ void token_embed(torch::Tensor out, torch::Tensor ids,
                  c10::optional<torch::Tensor> prev, torch::Tensor pos,
                  torch::Tensor embed, c10::optional<torch::Tensor> bigram,
                  long buckets, long mul_prev, long mul_cur,
-                 c10::optional<torch::Tensor> inv_freq) {
+                 c10::optional<torch::Tensor> inv_freq, double scale) {
   CHECK_GPU(out); CHECK_F32(out); CHECK_CONTIG(out); CHECK_GPU(ids);
   CHECK_I64(ids); CHECK_I64(pos); CHECK_CONTIG(ids); CHECK_CONTIG(pos);
   CHECK_GPU(embed); CHECK_CONTIG(embed);
@@ -394,8 +410,8 @@ void token_embed(torch::Tensor out, torch::Tensor ids,
   }
   mix_token_embed(out.data_ptr<float>(), ids.data_ptr<long>(), pp,
                   pos.data_ptr<long>(), embed.data_ptr(), bp, buckets,
-                  mul_prev, mul_cur, fp, T, (int)W, act_kind(embed),
-                  cur_stream());
+                  mul_prev, mul_cur, fp, (float)scale, T, (int)W,
+                  act_kind(embed), cur_stream());
 }
 
 void weighted_rmsnorm(torch::Tensor out, torch::Tensor x, torch::Tensor w,
@@ -599,6 +615,166 @@ void mlstm_out(torch::Tensor out, long out_off, torch::Tensor o,
                 cur_stream());
 }
 
+// ---- Dynamic-Tanh residual, routed experts, soft cap ----
+
+static const float* opt_f32(const c10::optional<torch::Tensor>& t, long n,
+                            const char* what) {
+  if (!t.has_value()) return nullptr;
+  TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kFloat &&
+              t->is_contiguous() && t->numel() == n, what,
+              ": fp32 GPU tensor of ", n, " values expected");
+  return t->data_ptr<float>();
+}
+
+void dyt_residual(torch::Tensor x, c10::optional<torch::Tensor> y1,
+                  c10::optional<torch::Tensor> ls1,
+                  c10::optional<torch::Tensor> y2,
+                  c10::optional<torch::Tensor> ls2,
+                  c10::optional<torch::Tensor> rows,
+                  c10::optional<torch::Tensor> padpos,
+                  c10::optional<torch::Tensor> wts,
+                  c10::optional<torch::Tensor> alpha,
+                  c10::optional<torch::Tensor> nw,
+                  c10::optional<torch::Tensor> nb,
+                  c10::optional<torch::Tensor> h_out) {
+  CHECK_GPU(x); CHECK_F32(x); CHECK_CONTIG(x);
+  TORCH_CHECK(x.dim() == 2, "x must be [T, W]");
+  const long T = x.size(0), W = x.size(1);
+  int kind = -1;
+  auto act = [&](const c10::optional<torch::Tensor>& t, long r, long c,
+                 const char* what) -> const void* {
+    if (!t.has_value()) return nullptr;
+    TORCH_CHECK(t->is_cuda() && t->is_contiguous() && t->dim() == 2 &&
+                (r < 0 || t->size(0) == r) && t->size(1) == c, what,
+                ": shape");
+    const int k = act_kind(*t);
+    TORCH_CHECK(kind < 0 || kind == k, "activation dtypes differ");
+    kind = k;
+    return t->data_ptr();
+  };
+  const void* y1p = act(y1, T, W, "y1");
+  const void* y2p = act(y2, T, W, "y2");
+  const void* rp = act(rows, -1, W, "rows");
+  const float* l1 = opt_f32(ls1, W, "ls1");
+  const float* l2 = opt_f32(ls2, W, "ls2");
+  TORCH_CHECK(!y1p || l1, "y1 needs ls1");
+  TORCH_CHECK(!(y2p || rp) || (y1p && l2), "a second branch needs y1 and ls2");
+  TORCH_CHECK(!(y2p && rp), "one second branch at most");
+  const int* pp = nullptr; const float* wp = nullptr; long k = 0;
+  if (rp) {
+    TORCH_CHECK(padpos.has_value() && wts.has_value(), "rows need padpos, wts");
+    CHECK_GPU(*padpos); CHECK_I32(*padpos); CHECK_CONTIG(*padpos);
+    CHECK_GPU(*wts); CHECK_F32(*wts); CHECK_CONTIG(*wts);
+    TORCH_CHECK(padpos->dim() == 2 && padpos->size(0) == T &&
+                wts->sizes() == padpos->sizes(), "padpos / wts must be [T, k]");
+    k = padpos->size(1);
+    pp = padpos->data_ptr<int>(); wp = wts->data_ptr<float>();
+  }
+  void* hp = nullptr;
+  const float* ap = nullptr; const float* nwp = nullptr; const float* nbp = nullptr;
+  if (h_out.has_value()) {
+    CHECK_GPU(*h_out); CHECK_CONTIG(*h_out);
+    TORCH_CHECK(h_out->dim() == 2 && h_out->size(0) == T && h_out->size(1) == W,
+                "h_out shape");
+    const int hk = act_kind(*h_out);
+    TORCH_CHECK(kind < 0 || kind == hk, "activation dtypes differ");
+    kind = hk;
+    hp = h_out->data_ptr();
+    ap = opt_f32(alpha, 1, "alpha");
+    nwp = opt_f32(nw, W, "norm weight");
+    nbp = opt_f32(nb, W, "norm bias");
+    TORCH_CHECK(ap && nwp && nbp, "h_out needs alpha, weight and bias");
+  }
+  if (kind < 0) return;   // nothing to do
+  mix_dyt_residual(x.data_ptr<float>(), y1p, l1, y2p, l2, rp, pp, wp, (int)k,
+                   ap, nwp, nbp, hp, T, (int)W, kind, cur_stream());
+}
+
+void moe_route(torch::Tensor idx, torch::Tensor wts, torch::Tensor logits,
+               long groups, long keep, long rank) {
+  CHECK_GPU(logits); CHECK_F32(logits); CHECK_CONTIG(logits);
+  CHECK_GPU(idx); CHECK_I32(idx); CHECK_CONTIG(idx);
+  CHECK_GPU(wts); CHECK_F32(wts); CHECK_CONTIG(wts);
+  TORCH_CHECK(logits.dim() == 2 && idx.dim() == 2, "router shapes");
+  const long T = logits.size(0), E = logits.size(1), top = idx.size(1);
+  TORCH_CHECK(idx.size(0) == T && wts.sizes() == idx.sizes(), "router shapes");
+  TORCH_CHECK(groups >= 1 && groups <= 1024 && E % groups == 0 && keep >= 1 &&
+              keep <= groups && rank >= 1, "router groups");
+  TORCH_CHECK(top >= 1 && top <= keep * (E / groups),
+              "more choices than the kept groups hold");
+  TORCH_CHECK(4 * (E + groups) * 4 <= 64 * 1024, "too many experts");
+  mix_moe_route(idx.data_ptr<int>(), wts.data_ptr<float>(),
+                logits.data_ptr<float>(), T, (int)E, (int)top, (int)groups,
+                (int)keep, (int)rank, cur_stream());
+}
+
+void moe_dispatch(torch::Tensor row_tok, torch::Tensor tile_off,
+                  torch::Tensor counts, torch::Tensor padpos,
+                  torch::Tensor idx, long bm) {
+  CHECK_GPU(idx); CHECK_I32(idx); CHECK_CONTIG(idx);
+  CHECK_GPU(row_tok); CHECK_I32(row_tok); CHECK_CONTIG(row_tok);
+  CHECK_GPU(tile_off); CHECK_I32(tile_off); CHECK_CONTIG(tile_off);
+  CHECK_GPU(counts); CHECK_I32(counts); CHECK_CONTIG(counts);
+  CHECK_GPU(padpos); CHECK_I32(padpos); CHECK_CONTIG(padpos);
+  TORCH_CHECK(idx.dim() == 2 && padpos.sizes() == idx.sizes(), "pair shapes");
+  const long T = idx.size(0), k = idx.size(1), E = counts.numel();
+  TORCH_CHECK(bm == 64 || bm == 128, "bm must be 64 or 128");
+  TORCH_CHECK(tile_off.numel() == E + 1 && row_tok.numel() % bm == 0 &&
+              row_tok.numel() >= T * k + E * (bm - 1), "segment table sizes");
+  TORCH_CHECK((2 * E + 1) * 4 <= 64 * 1024, "too many experts");
+  mix_moe_dispatch(row_tok.data_ptr<int>(), tile_off.data_ptr<int>(),
+                   counts.data_ptr<int>(), padpos.data_ptr<int>(),
+                   idx.data_ptr<int>(), T * k, (int)k, (int)E, (int)bm,
+                   row_tok.numel(), cur_stream());
+}
+
+void expert_gemm(torch::Tensor out, torch::Tensor a, torch::Tensor w,
+                 c10::optional<torch::Tensor> row_tok, torch::Tensor tile_off,
+                 torch::Tensor counts, long act, long bm) {
+  CHECK_GPU(a); CHECK_CONTIG(a); CHECK_GPU(w); CHECK_CONTIG(w);
+  CHECK_GPU(out); CHECK_CONTIG(out);
+  CHECK_I32(tile_off); CHECK_I32(counts); CHECK_GPU(tile_off); CHECK_GPU(counts);
+  TORCH_CHECK(w.dim() == 3 && a.dim() == 2 && out.dim() == 2, "operand ranks");
+  const long E = w.size(0), N = w.size(1), K = w.size(2);
+  const long n_rows = out.size(0);
+  TORCH_CHECK(bm == 64 || bm == 128, "bm must be 64 or 128");
+  TORCH_CHECK(act == 0 || act == 2, "activation: 0 (none) or 2 (relu squared)");
+  TORCH_CHECK(a.size(1) == K && out.size(1) == N && n_rows % bm == 0 &&
+              counts.numel() == E && tile_off.numel() == E + 1,
+              "operand shapes");
+  const int kind = act_kind(a);
+  TORCH_CHECK(act_kind(w) == kind && act_kind(out) == kind, "dtype mismatch");
+  const int* rt = nullptr;
+  if (row_tok.has_value()) {
+    CHECK_GPU(*row_tok); CHECK_I32(*row_tok); CHECK_CONTIG(*row_tok);
+    TORCH_CHECK(row_tok->numel() == n_rows, "row table size");
+    rt = row_tok->data_ptr<int>();
+  } else {
+    TORCH_CHECK(a.size(0) == n_rows, "a must be laid out in segments");
+  }
+  TORCH_CHECK((act == 2) == (rt != nullptr),
+              "the gathered stage carries the activation");
+  if (kind == 0 && K % 64 == 0 && N % 64 == 0) {
+    sutro_grouped_gemm(out.data_ptr(), a.data_ptr(), w.data_ptr(), rt,
+                       tile_off.data_ptr<int>(), counts.data_ptr<int>(), (int)E,
+                       (int)(n_rows / bm), (int)N, K, (int)act, (int)bm,
+                       cur_stream());
+    return;
+  }
+  mix_expert_gemm_plain(out.data_ptr(), a.data_ptr(), w.data_ptr(), rt,
+                        tile_off.data_ptr<int>(), counts.data_ptr<int>(),
+                        (int)E, (int)N, (int)K, (int)bm, n_rows,
+                        act == 2 ? 1 : 0, kind, cur_stream());
+}
+
+void softcap(torch::Tensor out, torch::Tensor z, double cap) {
+  CHECK_GPU(z); CHECK_CONTIG(z); CHECK_GPU(out); CHECK_F32(out);
+  CHECK_CONTIG(out);
+  TORCH_CHECK(out.numel() == z.numel() && cap > 0, "softcap operands");
+  mix_softcap(out.data_ptr<float>(), z.data_ptr(), (float)cap, z.numel(),
+              act_kind(z), cur_stream());
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("gelu_tanh_mul", &gelu_tanh_mul, "tanh-GELU(gate) * up");
   m.def("gated_norm_residual", &gated_norm_residual,
@@ -614,7 +790,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("gate_off"), py::arg("out_scale"),
         py::arg("tile_seq") = c10::nullopt, py::arg("tile_q0") = c10::nullopt,
         py::arg("prefill_rows") = 0, py::arg("bias_r1") = c10::nullopt,
-        py::arg("bias_r2") = c10::nullopt);
+        py::arg("bias_r2") = c10::nullopt, py::arg("sink") = false);
   m.def("delta_prep", &delta_prep, "delta-rule inputs: filters, norms, gates",
         py::arg("qn"), py::arg("kn"), py::arg("v"), py::arg("decay"),
         py::arg("beta"), py::arg("proj"), py::arg("q_off"), py::arg("k_off"),
@@ -626,7 +802,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("delta_scan", &delta_scan, "gated delta rule over new tokens");
   m.def("delta_out", &delta_out, "per-head norm + low-rank gate of the read-out");
   m.def("token_embed", &token_embed,
-        "token row + hashed-bigram row + position sinusoid, fp32");
+        "scaled token row + hashed-bigram row + position sinusoid, fp32",
+        py::arg("out"), py::arg("ids"), py::arg("prev"), py::arg("pos"),
+        py::arg("embed"), py::arg("bigram"), py::arg("buckets"),
+        py::arg("mul_prev"), py::arg("mul_cur"), py::arg("inv_freq"),
+        py::arg("scale") = 1.0);
   m.def("weighted_rmsnorm", &weighted_rmsnorm, "RMS norm with a weight vector");
   m.def("norm_residual", &norm_residual,
         "post-norm + residual (+ depth-weighted sum) (+ next pre-norm)");
@@ -638,4 +818,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("sigmoid_gate_mul", &sigmoid_gate_mul, "v *= sigmoid(gate section)");
   m.def("mlstm_scan", &mlstm_scan, "mLSTM memory over new tokens");
   m.def("mlstm_out", &mlstm_out, "mLSTM read-out normalisation, norm and gate");
+  m.def("dyt_residual", &dyt_residual,
+        "layer-scaled parallel residual (second branch dense or gathered "
+        "expert rows) + Dynamic-Tanh norm of the result");
+  m.def("moe_route", &moe_route,
+        "sigmoid router with group-limited choice and normalised weights");
+  m.def("moe_dispatch", &moe_dispatch,
+        "(token, choice) pairs -> padded per-expert segments");
+  m.def("expert_gemm", &expert_gemm,
+        "GEMM over padded per-expert segments (matrix cores for bf16 with "
+        "64-aligned sizes, plain tiles otherwise)");
+  m.def("softcap", &softcap, "cap * tanh(z / cap), fp32 out");
 }

@@ -1,5 +1,6 @@
 // Row-wise pieces of layer-list decoders that keep every layer's result:
-//   token_embed       X0 = token row + hashed-bigram row + position sinusoid
+//   token_embed       X0 = scale * token row + hashed-bigram row + position
+//                     sinusoid
 //   weighted_rmsnorm  h = n(x) * w
 //   norm_residual     r = x_in + n(y) * w_post -> x_out; optionally the
 //                     depth-weighted sum z = sum_j d[j] * X_j over the kept
@@ -18,7 +19,8 @@ __global__ void token_embed_kernel(
     float* __restrict__ out, const long* __restrict__ ids,
     const long* __restrict__ prev, const long* __restrict__ pos,
     const A* __restrict__ embed, const A* __restrict__ bigram, long buckets,
-    long mul_prev, long mul_cur, const float* __restrict__ inv_freq, int W) {
+    long mul_prev, long mul_cur, const float* __restrict__ inv_freq,
+    float scale, int W) {
   const long t = blockIdx.x;
   const long id = ids[t];
   const A* er = embed + id * W;
@@ -30,7 +32,7 @@ __global__ void token_embed_kernel(
   }
   const float p = (float)pos[t];
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    float x = ldf<A>(er + c);
+    float x = ldf<A>(er + c) * scale;
     if (br) x += ldf<A>(br + c);
     if (inv_freq) {
       const float ang = p * inv_freq[c >> 1];
@@ -265,19 +267,19 @@ extern "C" void mix_token_embed(float* out, const long* ids, const long* prev,
                                 const long* pos, const void* embed,
                                 const void* bigram, long buckets,
                                 long mul_prev, long mul_cur,
-                                const float* inv_freq, long T, int W, int f32,
-                                hipStream_t s) {
+                                const float* inv_freq, float scale, long T,
+                                int W, int f32, hipStream_t s) {
   if (T == 0) return;
   if (f32)
     hipLaunchKernelGGL(token_embed_kernel<float>, dim3((unsigned)T), dim3(256),
                        0, s, out, ids, prev, pos, (const float*)embed,
                        (const float*)bigram, buckets, mul_prev, mul_cur,
-                       inv_freq, W);
+                       inv_freq, scale, W);
   else
     hipLaunchKernelGGL(token_embed_kernel<u16>, dim3((unsigned)T), dim3(256), 0,
                        s, out, ids, prev, pos, (const u16*)embed,
                        (const u16*)bigram, buckets, mul_prev, mul_cur,
-                       inv_freq, W);
+                       inv_freq, scale, W);
 }
 
 extern "C" void mix_weighted_rmsnorm(void* out, const float* x, const float* w,

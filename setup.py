@@ -37,6 +37,9 @@ MIX_SOURCES = [
     "csrc/mix_stream.hip",
     "csrc/mix_prep.hip",
     "csrc/mix_mlstm.hip",
+    "csrc/mix_moe.hip",
+    # the matrix-core expert GEMM serves both extensions
+    "csrc/grouped_gemm.hip",
 ]
 
 # hipcc's automatic packed-fp32 forms are switched off for all device code

@@ -328,13 +328,14 @@ def moe_route(logits, top: int, groups: int, keep: int, group_rank: int = 2):
 
 def moe_dispatch(idx, experts: int, bm: int):
     """Per-expert segments padded to `bm` rows for idx int32 [T, k]:
-    (row_tok int32 [T*k + experts*bm], tile_off int32 [experts+1], counts
-    int32 [experts], padpos int32 [T, k]). One kernel, no host round trip."""
+    (row_tok int32 [(ceil(T*k / bm) + experts) * bm], tile_off int32
+    [experts+1], counts int32 [experts], padpos int32 [T, k]). One kernel, no
+    host round trip."""
     if idx.is_cuda:
         T, k = idx.shape
         dev = idx.device
-        row_tok = torch.empty(T * k + experts * bm, dtype=torch.int32,
-                              device=dev)
+        row_tok = torch.empty(((T * k + bm - 1) // bm + experts) * bm,
+                              dtype=torch.int32, device=dev)
         tile_off = torch.empty(experts + 1, dtype=torch.int32, device=dev)
         counts = torch.empty(experts, dtype=torch.int32, device=dev)
         padpos = torch.empty((T, k), dtype=torch.int32, device=dev)

@@ -635,7 +635,8 @@ def moe_route(logits, top: int, groups: int, keep: int, group_rank: int = 2):
 
 def moe_dispatch(idx, experts: int, bm: int):
     """Lay the (token, choice) pairs of idx [T, k] out in per-expert segments
-    padded to `bm` rows. Returns (row_tok int32 [T*k + experts*bm]: the token
+    padded to `bm` rows. Returns (row_tok int32 [(ceil(T*k / bm) + experts) *
+    bm], a whole number of tiles that holds every padded segment: the token
     of every padded row, -1 for padding; tile_off int32 [experts+1]: segment
     starts in tiles; counts int32 [experts]; padpos int32 [T, k]: the padded
     row of every pair)."""
@@ -652,8 +653,8 @@ def moe_dispatch(idx, experts: int, bm: int):
     se = flat[order]
     pos = torch.arange(T * k, device=dev) - first[se]
     where = pad_off[se] + pos
-    row_tok = torch.full((T * k + experts * bm,), -1, dtype=torch.int32,
-                         device=dev)
+    row_tok = torch.full((((T * k + bm - 1) // bm + experts) * bm,), -1,
+                         dtype=torch.int32, device=dev)
     row_tok[where] = (order // k).to(torch.int32)
     padpos = torch.empty(T * k, dtype=torch.int32, device=dev)
     padpos[order] = where.to(torch.int32)
