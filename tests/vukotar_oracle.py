@@ -57,8 +57,11 @@ def sink_attention(q, k, v, scale):
     return out
 
 
-def route(z, top, groups, keep):
+def route(z, top, groups, keep, gaps=None):
     """Router of one token. z [E] logits. Returns (chosen experts, weights).
+    `gaps`, when a list, gets how far the choice was from another one: the
+    distance between the worth of the last kept and the first dropped group,
+    and between the last chosen and the first unchosen allowed score.
     Scores are sigmoids. The experts form `groups` equal runs of neighbours; a
     group is worth the sum of its two largest scores (its only score if it has
     one expert); only experts of the `keep` best groups may be chosen; the
@@ -72,7 +75,14 @@ def route(z, top, groups, keep):
         worth.append(sum(part[:2]))
     best = sorted(range(groups), key=lambda g: (-worth[g], g))[:keep]
     allowed = [e for e in range(E) if e // size in best]
-    chosen = sorted(allowed, key=lambda e: (-float(s[e]), e))[:top]
+    ranked = sorted(allowed, key=lambda e: (-float(s[e]), e))
+    chosen = ranked[:top]
+    if gaps is not None:
+        by_worth = sorted(worth, reverse=True)
+        if keep < groups:
+            gaps.append(by_worth[keep - 1] - by_worth[keep])
+        if top < len(ranked):
+            gaps.append(float(s[ranked[top - 1]] - s[ranked[top]]))
     total = sum(float(s[e]) for e in chosen) + 1e-20
     return chosen, [float(s[e]) / total for e in chosen]
 
@@ -98,14 +108,14 @@ def attention_mixer(w, p, mc, h):
     return torch.cat(heads, dim=1) @ w[p + "o"].T
 
 
-def moe_feed_forward(w, p, fc, h, picks=None):
+def moe_feed_forward(w, p, fc, h, picks=None, gaps=None):
     r = fc["router"]
     E, top = r["experts"], r["top"]
     z = h @ w[p + "router"].T
     out = torch.zeros(h.shape[0], w[p + "e0.down"].shape[0], dtype=F64)
     for t in range(h.shape[0]):
         chosen, weights = route(z[t], top, r["groups"]["count"],
-                                r["groups"]["keep"])
+                                r["groups"]["keep"], gaps)
         if picks is not None:
             picks.append(chosen)
         for e, g in zip(chosen, weights):
@@ -120,10 +130,10 @@ def owner(config, i):
     return i
 
 
-def forward(config, w, tokens, streams=None, picks=None):
+def forward(config, w, tokens, streams=None, picks=None, gaps=None):
     """Logits [T, vocab] of one whole sequence. `streams`, when a list, gets
     the residual stream after every layer; `picks` the chosen experts of every
-    layer and token."""
+    layer and token; `gaps` how close every routing choice was (see route)."""
     W = config["width"]
     T = len(tokens)
     x = w["embed"][torch.tensor(tokens)] * config["embedding"]["scale"]
@@ -136,7 +146,7 @@ def forward(config, w, tokens, streams=None, picks=None):
         if layer_.get("mlp") is not None:
             mine = [] if picks is not None else None
             add = add + w[lp + "ls2"] * moe_feed_forward(
-                w, lp + "mlp.", layer_["mlp"], h, mine)
+                w, lp + "mlp.", layer_["mlp"], h, mine, gaps)
             if picks is not None:
                 picks.append(mine)
         x = x + add
@@ -191,7 +201,7 @@ def make_weights(config, seed=0):
     def norm(name):
         w[name] = rnd(W, std=0.2, mean=1.0)
         w[name + ".b"] = rnd(W, std=0.1)
-        w[name + ".alpha"] = rnd(std=0.05, mean=0.6)
+        w[name + ".alpha"] = rnd(1, std=0.05, mean=0.6)[0]
 
     w["embed"] = rnd(config["vocab"], W)
     norm("final.norm")
