@@ -74,13 +74,13 @@ def build_args():
                         "spawns one worker per GPU.")
     p.add_argument("--arch-compare", type=str, default=None, metavar="SIZES",
                    help="instead of the flagship workload: prefill and decode "
-                        "tokens/s of the Vodinex layer-list decoder beside "
-                        "the Qwen3 dense decoder of equal size, random "
-                        "weights (comma list of 1b,8b,tiny); one JSON line "
-                        "per model")
+                        "tokens/s of a layer-list decoder beside the Qwen3 "
+                        "decoder of equal size, random weights (comma list "
+                        "of 1b,8b,tiny); one JSON line per model")
     p.add_argument("--compare-models", type=str, default="vodinex,qwen3",
                    help="models of --arch-compare: comma list of vodinex, "
-                        "ruludra, qwen3")
+                        "ruludra, vukotar, qwen3, qwen3moe (vukotar's "
+                        "counterpart is qwen3moe)")
     p.add_argument("--compare-seqs", type=int, default=16)
     p.add_argument("--compare-prompt", type=int, default=2048)
     p.add_argument("--e2e-rows", type=int, default=3000,

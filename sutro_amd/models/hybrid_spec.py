@@ -468,7 +468,7 @@ def vukotar_spec(config: dict, name: str = "vukotar",
         norm_eps=float(config["norm"]["eps"]),
         max_context=int(config.get("max_context", 1 << 20)),
         checkpoint_dir=checkpoint_dir, pos_base=10000.0,
-        embed_scale=float(config["embedding"]["scale"]),
+        embed_scale=float((config.get("embedding") or {}).get("scale", 1.0)),
         logit_softcap=float(config.get("logit_softcap", 0.0) or 0.0),
         tie_embeddings=True,
         num_experts=max((l.moe.experts if l.moe else 0) for l in layers))

@@ -1,6 +1,8 @@
 """Prefill and decode throughput of the layer-list decoders (Vodinex,
-Ruludra) beside the Qwen3 dense decoder of equal size (same width, layers, heads, key/value heads, head
-size and feed-forward width), both with random weights, both through the
+Ruludra, Vukotar) beside the Qwen3 decoder of equal size (same width, layers,
+heads, key/value heads, head size and feed-forward width; for Vukotar the
+Qwen3 mixture-of-experts decoder with as many experts of the same inner
+width and as many choices a token), all with random weights, all through the
 engine's own batch path (scheduler, paged cache, state slots, decode
 hipGraphs). Used by `bench.py --arch-compare`.
 
@@ -21,7 +23,8 @@ from ..engine.engine import LLMEngine
 from ..models.hybrid_spec import (AttnMixerSpec, DeltaMixerSpec,
                                   HybridLayerSpec, HybridSpec,
                                   LatentAttnMixerSpec, MLSTMMixerSpec,
-                                  ParallelMixerSpec, TiedAttnMixerSpec)
+                                  ParallelMixerSpec, RoutedExpertsSpec,
+                                  TiedAttnMixerSpec)
 from ..models.registry import ModelSpec
 
 # name -> (width, layers, heads, kv_heads, head size, ff, vocab)
@@ -89,6 +92,44 @@ def sandwich_spec(name: str, window: int = 1024) -> HybridSpec:
                       pos_base=10000.0, logit_scale=0.5)
 
 
+# routed feed-forwards at a size: experts, choices a token, inner width as a
+# fraction of the dense feed-forward width
+MOE_EXPERTS, MOE_TOP, MOE_FF_DIV = 32, 4, 4
+
+
+def parallel_spec(name: str) -> HybridSpec:
+    """Vukotar at the same width, depth, heads and head size: every layer a
+    sink-softmax attention beside 32 squared-ReLU experts (8 groups of 4, the
+    best 4 groups stay, 4 experts a token, inner width ff/4); the second half
+    of the layers runs the parameters of the first half again."""
+    W, L, H, G, D, ff, V = SIZES[name]
+    attn = AttnMixerSpec(heads=H, kv_heads=G, dim=D, vdim=D, scale=D ** -0.5,
+                         qk_norm=False, bias=False, out_gate=False, sink=True)
+    moe = RoutedExpertsSpec(ff=max(64, ff // MOE_FF_DIV), experts=MOE_EXPERTS,
+                            top=MOE_TOP, groups=8, keep=4)
+    own = max(1, L // 2)
+    layers = [HybridLayerSpec("attention", attn, moe=moe,
+                              weights_of=None if i < own else i % own)
+              for i in range(L)]
+    return HybridSpec(name=f"vukotar-{name}", arch="vukotar", hidden_size=W,
+                      vocab_size=V, layers=tuple(layers), norm_eps=1e-6,
+                      max_context=1 << 20, pos_base=10000.0, embed_scale=0.5,
+                      logit_softcap=30.0, tie_embeddings=True,
+                      num_experts=MOE_EXPERTS)
+
+
+def moe_spec(name: str) -> ModelSpec:
+    """The Qwen3 mixture-of-experts decoder with as many experts of the same
+    inner width and as many choices a token (softmax router, SwiGLU
+    experts)."""
+    W, L, H, G, D, ff, V = SIZES[name]
+    return ModelSpec(name=f"qwen3moe-{name}", arch="qwen3_moe", hidden_size=W,
+                     num_layers=L, num_heads=H, num_kv_heads=G, head_dim=D,
+                     intermediate_size=ff, vocab_size=V, max_context=1 << 20,
+                     num_experts=MOE_EXPERTS, experts_per_token=MOE_TOP,
+                     moe_intermediate_size=max(64, ff // MOE_FF_DIV))
+
+
 def dense_spec(name: str) -> ModelSpec:
     W, L, H, G, D, ff, V = SIZES[name]
     return ModelSpec(name=f"qwen3-{name}", arch="qwen3", hidden_size=W,
@@ -148,7 +189,8 @@ def _measure(spec, device: str, seqs: int, prompt: int, steps: int,
 
 
 MAKERS = {"vodinex": hybrid_spec, "qwen3": dense_spec,
-          "ruludra": sandwich_spec}
+          "ruludra": sandwich_spec, "vukotar": parallel_spec,
+          "qwen3moe": moe_spec}
 
 
 def run_compare(sizes: List[str], device: str, seqs: int, prompt: int,
