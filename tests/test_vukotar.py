@@ -565,12 +565,14 @@ def test_router_choice_and_weights(backend, E, top, groups, keep):
 
 @pytest.mark.parametrize("T,W,ff,E,top", [(37, 44, 20, 6, 3), (5, 64, 128, 4, 2),
                                           (300, 128, 64, 16, 4), (1, 36, 8, 3, 3),
-                                          (700, 64, 64, 2, 1)])
+                                          (700, 64, 64, 2, 1),
+                                          (1100, 128, 128, 2, 2)])
 def test_expert_segments_and_gather(backend, T, W, ff, E, top):
     """Dispatch into padded per-expert segments, both expert GEMMs and the
     weighted gather inside the residual kernel against the oracle's experts,
-    token by token; sizes the matrix-core kernel takes and sizes it does not,
-    segments longer than one tile, experts nobody chose."""
+    token by token; sizes the matrix-core kernel takes (64- and 128-row
+    tiles, 64 and 128 columns a workgroup) and sizes it does not, segments
+    longer than one tile, experts nobody chose."""
     device, dtype = backend
     g = torch.Generator().manual_seed(T + W)
     h = (torch.randn(T, W, generator=g) * 0.7).to(dtype)
