@@ -305,13 +305,16 @@ __global__ void local_attention_kernel(
 // the value row. This is the kernel of single-token (decode) rows: with a
 // window of W keys a row costs W / (4 * 64 / LPR) dependent steps instead of
 // W. Needs dk and dv to be multiples of the 16-byte vector and at most
-// 64 vectors long; other shapes take the one-wave kernel above.
+// 64 vectors long; other shapes take the one-wave kernel above. NW waves a
+// workgroup: 4 when there are rows enough to fill the chip, 16 when few rows
+// face long contexts (a decode step of a small batch), so that every SIMD
+// still holds several waves with loads in flight.
 template <typename A> struct Vec16;
 template <> struct Vec16<u16> { typedef u16x8 type; };
 template <> struct Vec16<float> { typedef f32x4 type; };
 
-template <typename A, int LPR>
-__global__ void __launch_bounds__(256) local_attention_rows_kernel(
+template <typename A, int LPR, int NW>
+__global__ void __launch_bounds__(NW * 64) local_attention_rows_kernel(
     A* __restrict__ out, long ldo, int out_off, const A* __restrict__ q,
     const A* __restrict__ k_cache, const A* __restrict__ v_cache,
     const int* __restrict__ bt, int bt_stride, const int* __restrict__ seq_lens,
@@ -328,7 +331,7 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(
   constexpr int DP = LPR * EPL;           // padded row length
   constexpr int CS = 2 + DP;              // floats a wave leaves in LDS
   __shared__ float qs[DP];
-  __shared__ float comb[WPB * CS];
+  __shared__ float comb[NW * CS];
   const int lane = threadIdx.x & (WAVE - 1);
   const int wid = threadIdx.x / WAVE;
   const int kg = lane / LPR, c0 = (lane % LPR) * EPL;
@@ -359,7 +362,7 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(
   for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
 
   const int n_tiles = (p - lo) / TK + 1;
-  for (int tile = wid; tile < n_tiles; tile += WPB) {
+  for (int tile = wid; tile < n_tiles; tile += NW) {
     const int base = lo + tile * TK;
     float sc[TS];
     long vrow[TS];
@@ -436,12 +439,12 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(
   __syncthreads();
   float mx = comb[0];  // wave 0 always has a tile
 #pragma unroll
-  for (int w = 1; w < WPB; ++w) mx = fmaxf(mx, comb[w * CS]);
+  for (int w = 1; w < NW; ++w) mx = fmaxf(mx, comb[w * CS]);
   // a sink (score 0, no value) joins the normalisation here, once per row
   if (sink) mx = fmaxf(mx, 0.f);
-  float wgt[WPB], lsum = sink ? expf(-mx) : 0.f;
+  float wgt[NW], lsum = sink ? expf(-mx) : 0.f;
 #pragma unroll
-  for (int w = 0; w < WPB; ++w) {
+  for (int w = 0; w < NW; ++w) {
     wgt[w] = expf(comb[w * CS] - mx);   // a wave without tiles: exp(-inf) = 0
     lsum += wgt[w] * comb[w * CS + 1];
   }
@@ -451,7 +454,7 @@ __global__ void __launch_bounds__(256) local_attention_rows_kernel(
   for (int c = threadIdx.x; c < dv; c += blockDim.x) {
     float o = 0.f;
 #pragma unroll
-    for (int w = 0; w < WPB; ++w) o += wgt[w] * comb[w * CS + 2 + c];
+    for (int w = 0; w < NW; ++w) o += wgt[w] * comb[w * CS + 2 + c];
     stf<A>(out + t * ldo + out_off + (long)h * dv + c, o * f);
   }
 }
@@ -516,9 +519,16 @@ static void launch_local_attention(
     if (dk % EPL == 0 && dv % EPL == 0 && dmax <= 64 * EPL) {
       int lpr = 2;
       while (lpr * EPL < dmax) lpr <<= 1;
+      // few rows over long tables (the table width bounds the context)
+      const bool wide = units <= 512 && (long)bt_stride * page >= 512;
 #define LAUNCH_LR(LL)                                                         \
-  hipLaunchKernelGGL((local_attention_rows_kernel<A, LL>),                    \
-                     dim3((unsigned)units), dim3(WPB * WAVE), 0, s, (A*)out,  \
+  do {                                                                        \
+    if (wide) LAUNCH_LRN(LL, 16);                                             \
+    else LAUNCH_LRN(LL, 4);                                                   \
+  } while (0)
+#define LAUNCH_LRN(LL, NN)                                                    \
+  hipLaunchKernelGGL((local_attention_rows_kernel<A, LL, NN>),                \
+                     dim3((unsigned)units), dim3(NN * WAVE), 0, s, (A*)out,   \
                      ldo, out_off, (const A*)q, (const A*)k_cache,            \
                      (const A*)v_cache, bt, bt_stride, seq_lens, qlocs,       \
                      token_seq, scale, chunk, window, (const A*)proj, ld,     \
@@ -531,6 +541,7 @@ static void launch_local_attention(
       else if (lpr == 32) LAUNCH_LR(32);
       else LAUNCH_LR(64);
 #undef LAUNCH_LR
+#undef LAUNCH_LRN
       return;
     }
   }

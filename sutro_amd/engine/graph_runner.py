@@ -105,6 +105,23 @@ class DecodeGraphRunner:
 
     @torch.no_grad()
     def _capture_all(self) -> None:
+        """Python's cyclic collector stays off while streams capture: it runs
+        at arbitrary allocations, and when it then frees an engine that is no
+        longer referenced (its graphs, pools and events) the runtime refuses
+        those calls inside a capture and the process aborts. Dead objects are
+        collected once before the captures instead."""
+        import gc
+
+        gc.collect()
+        was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            self._capture_buckets()
+        finally:
+            if was_enabled:
+                gc.enable()
+
+    def _capture_buckets(self) -> None:
         eng = self.engine
         torch.cuda.synchronize()
         self._pool = torch.cuda.graph_pool_handle()

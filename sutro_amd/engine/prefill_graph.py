@@ -95,8 +95,19 @@ class PrefillGraphRunner:
             ctx = torch.cuda.graph(g, pool=pool)
         else:
             ctx = torch.cuda.graph(g)
-        with ctx:
-            hidden = eng.model(self._fb, eng.kv)
+        # no cyclic collection inside the capture: freeing a dead engine's
+        # graphs or events there is refused by the runtime and aborts
+        import gc
+
+        gc.collect()
+        was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            with ctx:
+                hidden = eng.model(self._fb, eng.kv)
+        finally:
+            if was_enabled:
+                gc.enable()
         self.graph = g
         self.hidden_out = hidden
         torch.cuda.synchronize()

@@ -415,7 +415,9 @@ def test_decode_graph_replays_equal_eager_steps(tmp_path_factory, dtype):
     """Single-token steps run as captured hipGraphs (router, dispatch, expert
     GEMMs and the gather inside). Many replays with prompt pieces of other
     requests and host synchronisation between them must give, every time,
-    what an engine that captures nothing gives."""
+    what an engine that captures nothing gives (up to rounding: a graph pads
+    its batch and its block tables, so GEMMs and the decode attention may sum
+    in another order)."""
     ck = checkpoint(tmp_path_factory, "config_c", config_c)
     seqs = {"a": tokens_for(ck[1], 60, 1), "b": tokens_for(ck[1], 45, 2),
             "c": tokens_for(ck[1], 38, 3)}
@@ -428,7 +430,38 @@ def test_decode_graph_replays_equal_eager_steps(tmp_path_factory, dtype):
     assert eager.graph_runner is None
     got, want = replay(graphs, seqs, schedule), replay(eager, seqs, schedule)
     for k in seqs:
-        assert torch.equal(got[k], want[k]), k
+        rows = row_errors(got[k], want[k].double().cpu())
+        if dtype == torch.float32:
+            assert float(rows.max()) < 1e-5, (k, float(rows.max()))
+        else:
+            assert float(rows.median()) < 2e-2, (k, float(rows.median()))
+            assert int((rows > 0.3).sum()) <= max(1, len(rows) // 10), k
+
+
+@pytest.mark.gpu
+def test_no_cyclic_collection_inside_graph_captures(tmp_path_factory, monkeypatch):
+    """Python's cyclic collector must be off while a stream captures: it runs
+    at arbitrary allocations, and freeing an unreferenced engine's graphs and
+    events inside a capture is refused by the runtime. After the captures it
+    is on again."""
+    import gc
+
+    from sutro_amd.models.vukotar import VukotarModel
+
+    seen = []
+    plain = VukotarModel.forward
+
+    def watched(self, fb, kv):
+        seen.append((torch.cuda.is_current_stream_capturing(), gc.isenabled()))
+        return plain(self, fb, kv)
+
+    monkeypatch.setattr(VukotarModel, "forward", watched)
+    ck = checkpoint(tmp_path_factory, "config_b", config_b)
+    assert gc.isenabled()
+    eng = engine(ck, ("cuda", torch.float32))
+    assert eng.graph_runner is not None and gc.isenabled()
+    captured = [on for capturing, on in seen if capturing]
+    assert captured and not any(captured)
 
 
 # ------------------------------------------------- mechanisms on their own --
