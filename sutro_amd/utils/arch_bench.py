@@ -113,8 +113,8 @@ def parallel_spec(name: str) -> HybridSpec:
               for i in range(L)]
     return HybridSpec(name=f"vukotar-{name}", arch="vukotar", hidden_size=W,
                       vocab_size=V, layers=tuple(layers), norm_eps=1e-6,
-                      max_context=1 << 20, pos_base=10000.0, embed_scale=0.5,
-                      logit_softcap=30.0, tie_embeddings=True,
+                      max_context=1 << 20, pos_base=10000.0, embed_scale=0.7,
+                      logit_softcap=25.0, tie_embeddings=True,
                       num_experts=MOE_EXPERTS)
 
 
