@@ -92,6 +92,8 @@ __device__ __forceinline__ const bf16x8* gg_frag(const u16* lds, int row,
 // MODE=1: rows gathered, B has two streams (gate/up at N-offset 0 and n_cols), output
 // n_cols wide with silu(g)*u. MODE=0: plain A, plain B, plain store.
 // MODE=2: rows gathered, one B stream, relu(x)^2 in the epilogue.
+// MODE=3: like MODE=1 with the clamped unit g sigmoid(1.702 g) (u + 1),
+// g = min(gate, limit), u = clamp(up, -limit, limit).
 // Waves arranged WROWS(M) x WCOLS(N); wave tile = (BM/WROWS) x (BN/WCOLS).
 template <int MODE, int BM, int BN, int WROWS, int WCOLS>
 __global__ __launch_bounds__(WROWS* WCOLS * 64) void grouped_gemm_kernel(
@@ -101,8 +103,8 @@ __global__ __launch_bounds__(WROWS* WCOLS * 64) void grouped_gemm_kernel(
     const int* __restrict__ row_tok,    // [rows_max] or nullptr
     const int* __restrict__ tile_off,   // [E+1] padded-offset / BM
     const int* __restrict__ counts,     // [E] live rows per expert
-    int n_experts, int n_cols, long K) {
-  constexpr bool GATED = MODE == 1;   // silu(gate) * up over two B streams
+    int n_experts, int n_cols, long K, float limit) {
+  constexpr bool GATED = MODE == 1 || MODE == 3;  // two B streams (gate, up)
   constexpr bool GATHER = MODE != 0;  // A rows come through row_tok
   constexpr int WAVES = WROWS * WCOLS;
   constexpr int WM = BM / WROWS;
@@ -128,7 +130,7 @@ __global__ __launch_bounds__(WROWS* WCOLS * 64) void grouped_gemm_kernel(
   const int wave = threadIdx.x >> 6;
   const int wm = wave / WCOLS, wn = wave % WCOLS;
 
-  __shared__ u16 smem[2][(BM + (MODE == 1 ? 2 : 1) * BN) * 64];
+  __shared__ u16 smem[2][(BM + (GATED ? 2 : 1) * BN) * 64];
   const int b_off = BM * 64;
   const int b2_off = (BM + BN) * 64;
 
@@ -218,9 +220,14 @@ __global__ __launch_bounds__(WROWS* WCOLS * 64) void grouped_gemm_kernel(
         const int grow = grow0 + r;
         const long o = (long)(seg0 + m0 + grow) * n_cols + gn;
         float v = accg[i][j][r];
-        if (GATED) {
+        if (MODE == 1) {
           const float g = v;
           v = g / (1.0f + __expf(-g)) * accu[i][j][r];
+        }
+        if (MODE == 3) {
+          const float g = fminf(v, limit);
+          const float u = fminf(fmaxf(accu[i][j][r], -limit), limit);
+          v = g / (1.0f + __expf(-1.702f * g)) * (u + 1.0f);
         }
         if (MODE == 2) {
           v = fmaxf(v, 0.f);
@@ -232,12 +239,12 @@ __global__ __launch_bounds__(WROWS* WCOLS * 64) void grouped_gemm_kernel(
   }
 }
 
-extern "C" void sutro_grouped_gemm(void* out, const void* a, const void* w,
-                                   const int* row_tok, const int* tile_off,
-                                   const int* counts, int n_experts,
-                                   int max_tiles, int n_cols, long K,
-                                   int gate_silu, int bm,
-                                   hipStream_t stream) {
+static void grouped_gemm_launch(void* out, const void* a, const void* w,
+                                const int* row_tok, const int* tile_off,
+                                const int* counts, int n_experts,
+                                int max_tiles, int n_cols, long K,
+                                int gate_silu, int bm, float limit,
+                                hipStream_t stream) {
   if (max_tiles == 0) return;
 #define GG_LAUNCH(GS, BM, BN, WR, WC)                                       \
   {                                                                         \
@@ -246,25 +253,49 @@ extern "C" void sutro_grouped_gemm(void* out, const void* a, const void* w,
     hipLaunchKernelGGL((grouped_gemm_kernel<GS, BM, BN, WR, WC>), grid,     \
                        block, 0, stream, (u16*)out, (const u16*)a,          \
                        (const u16*)w, row_tok, tile_off, counts, n_experts, \
-                       n_cols, K);                                          \
+                       n_cols, K, limit);                                   \
     return;                                                                 \
   }
   /* no hipGetLastError in this launcher: error-state queries are rejected
      while a stream is capturing (decode steps replay under hipGraphs) */
   if (bm == 128 && n_cols % 128 == 0) {
     if (gate_silu == 1) GG_LAUNCH(1, 128, 128, 2, 4)
+    else if (gate_silu == 3) GG_LAUNCH(3, 128, 128, 2, 4)
     else if (gate_silu == 2) GG_LAUNCH(2, 128, 128, 2, 4)
     else GG_LAUNCH(0, 128, 128, 2, 4)
   }
   if (bm == 128) {
     if (gate_silu == 1) GG_LAUNCH(1, 128, 64, 4, 2)
+    else if (gate_silu == 3) GG_LAUNCH(3, 128, 64, 4, 2)
     else if (gate_silu == 2) GG_LAUNCH(2, 128, 64, 4, 2)
     else GG_LAUNCH(0, 128, 64, 4, 2)
   }
   if (gate_silu == 1) GG_LAUNCH(1, 64, 64, 2, 2)
+  else if (gate_silu == 3) GG_LAUNCH(3, 64, 64, 2, 2)
   else if (gate_silu == 2) GG_LAUNCH(2, 64, 64, 2, 2)
   else GG_LAUNCH(0, 64, 64, 2, 2)
 #undef GG_LAUNCH
+}
+
+extern "C" void sutro_grouped_gemm(void* out, const void* a, const void* w,
+                                   const int* row_tok, const int* tile_off,
+                                   const int* counts, int n_experts,
+                                   int max_tiles, int n_cols, long K,
+                                   int gate_silu, int bm,
+                                   hipStream_t stream) {
+  grouped_gemm_launch(out, a, w, row_tok, tile_off, counts, n_experts,
+                      max_tiles, n_cols, K, gate_silu, bm, 0.f, stream);
+}
+
+// the clamped gated unit (mode 3) with its limit
+extern "C" void sutro_grouped_gemm_glu(void* out, const void* a, const void* w,
+                                       const int* row_tok, const int* tile_off,
+                                       const int* counts, int n_experts,
+                                       int max_tiles, int n_cols, long K,
+                                       int bm, float limit,
+                                       hipStream_t stream) {
+  grouped_gemm_launch(out, a, w, row_tok, tile_off, counts, n_experts,
+                      max_tiles, n_cols, K, 3, bm, limit, stream);
 }
 
 // ---- fused MoE combine: out[t] = sum_j w[t,j] * rows[padpos[t,j]] ----

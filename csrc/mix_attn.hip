@@ -38,7 +38,9 @@ __global__ void attn_prep_kernel(
     const float* __restrict__ k_w, float eps,
     const float* __restrict__ cos_sin, int half,
     const long* __restrict__ slots, A* __restrict__ k_cache,
-    A* __restrict__ v_cache, long T, int H, int G, int dk, int dv, int page) {
+    A* __restrict__ v_cache, const A* __restrict__ vfirst, long ldvf,
+    const float* __restrict__ vlam, long T, int H, int G, int dk, int dv,
+    int page) {
   extern __shared__ float sm[];  // WPB * dmax floats
   const int lane = threadIdx.x & (WAVE - 1);
   const int wid = threadIdx.x / WAVE;
@@ -64,6 +66,16 @@ __global__ void attn_prep_kernel(
     for (int k = 0; k < DPL; ++k) {
       const int i = lane + k * (int)WAVE;
       x[n][k] = i < d ? ldf<A>(src + i) : 0.f;
+    }
+    if (vfirst && kind == 2) {
+      // cached value = (1 - lambda) v + lambda * (another layer's value)
+      const float lam = vlam[0];
+      const A* vf = vfirst + t * ldvf + (long)head * d;
+#pragma unroll
+      for (int k = 0; k < DPL; ++k) {
+        const int i = lane + k * (int)WAVE;
+        if (i < d) x[n][k] = (1.f - lam) * x[n][k] + lam * ldf<A>(vf + i);
+      }
     }
   }
 #pragma unroll
@@ -130,7 +142,9 @@ __global__ void attn_prep_vec_kernel(
     const float* __restrict__ k_w, float eps,
     const float* __restrict__ cos_sin, int half,
     const long* __restrict__ slots, u16* __restrict__ k_cache,
-    u16* __restrict__ v_cache, long T, int H, int G, int dk, int dv, int page) {
+    u16* __restrict__ v_cache, const u16* __restrict__ vfirst, long ldvf,
+    const float* __restrict__ vlam, long T, int H, int G, int dk, int dv,
+    int page) {
   constexpr int UPWV = 64 / GS;
   const int lane = threadIdx.x & (WAVE - 1);
   const int wid = threadIdx.x / WAVE;
@@ -154,6 +168,13 @@ __global__ void attn_prep_vec_kernel(
     u16x8 raw = (u16x8)(0);
     if (act) raw = *(const u16x8*)src;
     bf8_to_f32(raw, x);
+    if (vfirst && kind == 2 && act) {
+      const float lam = vlam[0];
+      float y[8];
+      bf8_to_f32(*(const u16x8*)(vfirst + t * ldvf + (long)head * d + c0), y);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = (1.f - lam) * x[e] + lam * y[e];
+    }
   }
   float ssq = 0.f;
 #pragma unroll
@@ -216,7 +237,7 @@ __global__ void local_attention_kernel(
     const int* __restrict__ qlocs, const int* __restrict__ token_seq,
     float scale, int chunk, int window, const A* __restrict__ proj, long ld,
     int gate_off, float out_scale, const float* __restrict__ bias_r1,
-    const float* __restrict__ bias_r2, int sink, long t0, long T, int H, int G,
+    const float* __restrict__ bias_r2, int sink, int keep_first, long t0, long T, int H, int G,
     int dk, int dv, int page) {
   extern __shared__ float sm[];  // WPB * dk floats: the wave's query
   const int lane = threadIdx.x & (WAVE - 1);
@@ -236,7 +257,12 @@ __global__ void local_attention_kernel(
   const int p = seq_lens[s] - (qlocs[s + 1] - (int)t);  // position of token t
   int lo = 0;
   if (chunk > 0) lo = (p / chunk) * chunk;
+  const int clo = lo;
   if (window > 0 && p - window + 1 > lo) lo = p - window + 1;
+  // kept first keys [clo, min(keep_first, lo)) come before the window: the
+  // loop runs over virtual indices vlo..p, the first nk of which are kept keys
+  const int nk = max(min(keep_first, lo) - clo, 0);
+  const int vlo = lo - nk;
   const int* table = bt + (long)s * bt_stride;
   // distance bias: r1 * ln(1 + r2 * (p - j)) is taken off the score
   const float r1 = bias_r1 ? bias_r1[h] : 0.f;
@@ -248,9 +274,10 @@ __global__ void local_attention_kernel(
 #pragma unroll
   for (int c = 0; c < NV; ++c) acc[c] = 0.f;
 
-  for (int base = lo; base <= p; base += WAVE) {
-    const int j = base + lane;
-    const bool live = j <= p;
+  for (int base = vlo; base <= p; base += WAVE) {
+    const int jv = base + lane;
+    const bool live = jv <= p;
+    const int j = jv - vlo < nk ? clo + (jv - vlo) : jv;
     int row = 0;  // blk * page + offset of key j
     float sc = -INFINITY;
     if (live) {
@@ -321,7 +348,7 @@ __global__ void __launch_bounds__(NW * 64) local_attention_rows_kernel(
     const int* __restrict__ qlocs, const int* __restrict__ token_seq,
     float scale, int chunk, int window, const A* __restrict__ proj, long ld,
     int gate_off, float out_scale, const float* __restrict__ bias_r1,
-    const float* __restrict__ bias_r2, int sink, long t0, int H, int G, int dk,
+    const float* __restrict__ bias_r2, int sink, int keep_first, long t0, int H, int G, int dk,
     int dv, int page) {
   typedef typename Vec16<A>::type vec_t;
   constexpr int EPL = 16 / sizeof(A);     // elements per lane
@@ -350,7 +377,12 @@ __global__ void __launch_bounds__(NW * 64) local_attention_rows_kernel(
   const int p = seq_lens[s] - (qlocs[s + 1] - (int)t);  // position of token t
   int lo = 0;
   if (chunk > 0) lo = (p / chunk) * chunk;
+  const int clo = lo;
   if (window > 0 && p - window + 1 > lo) lo = p - window + 1;
+  // kept first keys [clo, min(keep_first, lo)) take the first nk virtual
+  // indices of vlo..p
+  const int nk = max(min(keep_first, lo) - clo, 0);
+  const int vlo = lo - nk;
   const int* table = bt + (long)s * bt_stride;
   const float r1 = bias_r1 ? bias_r1[h] : 0.f;
   const float r2 = bias_r1 ? bias_r2[h] : 0.f;
@@ -361,16 +393,17 @@ __global__ void __launch_bounds__(NW * 64) local_attention_rows_kernel(
 #pragma unroll
   for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
 
-  const int n_tiles = (p - lo) / TK + 1;
+  const int n_tiles = (p - vlo) / TK + 1;
   for (int tile = wid; tile < n_tiles; tile += NW) {
-    const int base = lo + tile * TK;
+    const int base = vlo + tile * TK;
     float sc[TS];
     long vrow[TS];
     float tmax = -INFINITY;
 #pragma unroll
     for (int st = 0; st < TS; ++st) {
-      const int j = base + st * KPI + kg;
-      const bool live = j <= p;
+      const int jv = base + st * KPI + kg;
+      const bool live = jv <= p;
+      const int j = jv - vlo < nk ? clo + (jv - vlo) : jv;
       float dot = 0.f;
       long cell = 0;  // (blk * G + g) * page + off
       if (live) {
@@ -464,6 +497,8 @@ extern "C" void mix_attn_prep(void* q_out, const void* proj, long ld,
                               const float* q_w, const float* k_w, float eps,
                               const float* cos_sin, int half,
                               const long* slots, void* k_cache, void* v_cache,
+                              const void* vfirst, long ldvf,
+                              const float* vlam,
                               long T, int H, int G, int dk, int dv, int page,
                               int f32, hipStream_t s) {
   const long units = (T * (H + 2 * G) + UPW - 1) / UPW;
@@ -472,7 +507,9 @@ extern "C" void mix_attn_prep(void* q_out, const void* proj, long ld,
   const size_t smem = (size_t)WPB * dmax * sizeof(float);
   if (grid == 0) return;
   const int dm8 = (dmax + 7) / 8;
+  // vfirst points at the first value column: 16-byte loads need it aligned
   if (!f32 && dk % 8 == 0 && dv % 8 == 0 && half % 8 == 0 && ld % 8 == 0 &&
+      (!vfirst || (ldvf % 8 == 0 && ((size_t)vfirst & 15) == 0)) &&
       q_off % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 && dm8 <= 32) {
     const int GS = dm8 <= 4 ? 4 : (dm8 <= 8 ? 8 : (dm8 <= 16 ? 16 : 32));
     const long tot = T * (H + 2 * G);
@@ -482,7 +519,8 @@ extern "C" void mix_attn_prep(void* q_out, const void* proj, long ld,
   hipLaunchKernelGGL(attn_prep_vec_kernel<GG>, dim3(vgrid), dim3(WPB * WAVE), \
                      0, s, (u16*)q_out, (const u16*)proj, ld, q_off, k_off,   \
                      v_off, q_w, k_w, eps, cos_sin, half, slots,              \
-                     (u16*)k_cache, (u16*)v_cache, T, H, G, dk, dv, page)
+                     (u16*)k_cache, (u16*)v_cache, (const u16*)vfirst, ldvf,  \
+                     vlam, T, H, G, dk, dv, page)
     if (GS == 4) LAUNCH_PV(4);
     else if (GS == 8) LAUNCH_PV(8);
     else if (GS == 16) LAUNCH_PV(16);
@@ -494,12 +532,14 @@ extern "C" void mix_attn_prep(void* q_out, const void* proj, long ld,
     hipLaunchKernelGGL(attn_prep_kernel<float>, dim3(grid), dim3(WPB * WAVE),
                        smem, s, (float*)q_out, (const float*)proj, ld, q_off,
                        k_off, v_off, q_w, k_w, eps, cos_sin, half, slots,
-                       (float*)k_cache, (float*)v_cache, T, H, G, dk, dv, page);
+                       (float*)k_cache, (float*)v_cache, (const float*)vfirst,
+                       ldvf, vlam, T, H, G, dk, dv, page);
   else
     hipLaunchKernelGGL(attn_prep_kernel<u16>, dim3(grid), dim3(WPB * WAVE),
                        smem, s, (u16*)q_out, (const u16*)proj, ld, q_off,
                        k_off, v_off, q_w, k_w, eps, cos_sin, half, slots,
-                       (u16*)k_cache, (u16*)v_cache, T, H, G, dk, dv, page);
+                       (u16*)k_cache, (u16*)v_cache, (const u16*)vfirst, ldvf,
+                       vlam, T, H, G, dk, dv, page);
 }
 
 template <typename A>
@@ -508,7 +548,8 @@ static void launch_local_attention(
     const void* v_cache, const int* bt, int bt_stride, const int* seq_lens,
     const int* qlocs, const int* token_seq, float scale, int chunk,
     int window, const void* proj, long ld, int gate_off, float out_scale,
-    const float* bias_r1, const float* bias_r2, int sink, long t0, long T,
+    const float* bias_r1, const float* bias_r2, int sink, int keep_first,
+    long t0, long T,
     int H, int G, int dk, int dv, int page, hipStream_t s) {
   const long units = T * H;
   const int grid = (int)((units + WPB - 1) / WPB);
@@ -532,7 +573,7 @@ static void launch_local_attention(
                      ldo, out_off, (const A*)q, (const A*)k_cache,            \
                      (const A*)v_cache, bt, bt_stride, seq_lens, qlocs,       \
                      token_seq, scale, chunk, window, (const A*)proj, ld,     \
-                     gate_off, out_scale, bias_r1, bias_r2, sink, t0, H, G,   \
+                     gate_off, out_scale, bias_r1, bias_r2, sink, keep_first, t0, H, G,   \
                      dk, dv, page)
       if (lpr == 2) LAUNCH_LR(2);
       else if (lpr == 4) LAUNCH_LR(4);
@@ -552,7 +593,7 @@ static void launch_local_attention(
                      (const A*)q, (const A*)k_cache, (const A*)v_cache, bt,  \
                      bt_stride, seq_lens, qlocs, token_seq, scale, chunk,    \
                      window, (const A*)proj, ld, gate_off, out_scale,        \
-                     bias_r1, bias_r2, sink, t0, T, H, G, dk, dv, page)
+                     bias_r1, bias_r2, sink, keep_first, t0, T, H, G, dk, dv, page)
   if (dv <= 64) LAUNCH_LA(1);
   else if (dv <= 128) LAUNCH_LA(2);
   else if (dv <= 256) LAUNCH_LA(4);
@@ -565,18 +606,19 @@ extern "C" void mix_local_attention(
     const void* v_cache, const int* bt, int bt_stride, const int* seq_lens,
     const int* qlocs, const int* token_seq, float scale, int chunk,
     int window, const void* proj, long ld, int gate_off, float out_scale,
-    const float* bias_r1, const float* bias_r2, int sink, long t0, long T,
+    const float* bias_r1, const float* bias_r2, int sink, int keep_first,
+    long t0, long T,
     int H, int G, int dk, int dv, int page, int f32, hipStream_t s) {
   if (f32)
     launch_local_attention<float>(out, ldo, out_off, q, k_cache, v_cache, bt,
                                   bt_stride, seq_lens, qlocs, token_seq, scale,
                                   chunk, window, proj, ld, gate_off, out_scale,
-                                  bias_r1, bias_r2, sink, t0, T, H, G, dk, dv,
+                                  bias_r1, bias_r2, sink, keep_first, t0, T, H, G, dk, dv,
                                   page, s);
   else
     launch_local_attention<u16>(out, ldo, out_off, q, k_cache, v_cache, bt,
                                 bt_stride, seq_lens, qlocs, token_seq, scale,
                                 chunk, window, proj, ld, gate_off, out_scale,
-                                bias_r1, bias_r2, sink, t0, T, H, G, dk, dv,
+                                bias_r1, bias_r2, sink, keep_first, t0, T, H, G, dk, dv,
                                 page, s);
 }

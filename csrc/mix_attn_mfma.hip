@@ -53,7 +53,7 @@ local_attention_mfma_kernel(
     const int* __restrict__ tile_q0, float scale, int chunk, int window,
     const u16* __restrict__ proj, long ld, int gate_off, float out_scale,
     const float* __restrict__ bias_r1, const float* __restrict__ bias_r2,
-    int sink, int H, int Hk, int dk, int dv, int parts) {
+    int sink, int keep_first, int H, int Hk, int dk, int dv, int parts) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int w = threadIdx.x / WAVE;
   const int G = blockDim.x / WAVE;        // query heads of this workgroup
@@ -82,9 +82,11 @@ local_attention_mfma_kernel(
   const int my_p = p0 + my_q;             // position of this lane's query row
   int lo_row = 0;
   if (chunk > 0) lo_row = (my_p / chunk) * chunk;
+  const int clo_row = lo_row;             // kept first keys: [clo_row, keep_first)
   if (window > 0) lo_row = max(lo_row, my_p - window + 1);
   int lo_tile = 0;                        // bound of the tile's first row
   if (chunk > 0) lo_tile = (p0 / chunk) * chunk;
+  const int clo_tile = lo_tile;
   if (window > 0) lo_tile = max(lo_tile, p0 - window + 1);
 
   bfrag qb[DKP / 16];
@@ -108,7 +110,11 @@ local_attention_mfma_kernel(
   const float r2 = bias_r1 ? bias_r2[hq] : 0.f;
 
   const int kt0 = lo_tile / PG, kt1 = (kv_end + PG - 1) / PG;
-  for (int kt = kt0; kt < kt1; ++kt) {
+  // pages of kept first keys that lie wholly before the window's pages
+  const int kf0 = clo_tile / PG;
+  const int n_kept = max(min(kt0, (keep_first + PG - 1) / PG) - kf0, 0);
+  for (int it = 0; it < n_kept + kt1 - kt0; ++it) {
+    const int kt = it < n_kept ? kf0 + it : kt0 + (it - n_kept);
     const int blk = bt[(long)s * bt_stride + kt];
     const u16* kp = k_cache + (((long)blk * Hk + kh) * PG) * dk;
     const u16* vp = v_cache + (((long)blk * Hk + kh) * PG) * dv;
@@ -146,7 +152,8 @@ local_attention_mfma_kernel(
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int kvpos = kv0 + drow(r, hi);
-      vis[r] = kvpos <= my_p && kvpos >= lo_row;
+      vis[r] = kvpos <= my_p &&
+               (kvpos >= lo_row || (kvpos < keep_first && kvpos >= clo_row));
       float sv = d1[r] * scale;
       if (bias_r1) sv -= r1 * logf(1.f + r2 * (float)max(my_p - kvpos, 0));
       sc[r] = vis[r] ? sv : -1e30f;
@@ -227,7 +234,8 @@ extern "C" int mix_local_attention_mfma(
     const int* qlocs, const int* tile_seq, const int* tile_q0, int n_tiles,
     float scale, int chunk, int window, const void* proj, long ld,
     int gate_off, float out_scale, const float* bias_r1, const float* bias_r2,
-    int sink, int H, int Hk, int dk, int dv, int page, hipStream_t s) {
+    int sink, int keep_first, int H, int Hk, int dk, int dv, int page,
+    hipStream_t s) {
   if (page != PG || dk % 8 || dv % 8 || dk > 256 || dv > 256 || H % Hk)
     return 0;
   const int DKP = dk <= 64 ? 64 : (dk <= 128 ? 128 : 256);
@@ -253,7 +261,7 @@ extern "C" int mix_local_attention_mfma(
                      (const u16*)v_cache, bt, bt_stride, seq_lens, qlocs,     \
                      tile_seq, tile_q0, scale, chunk, window,                 \
                      (const u16*)proj, ld, gate_off, out_scale, bias_r1,     \
-                     bias_r2, sink, H, Hk, dk, dv, parts)
+                     bias_r2, sink, keep_first, H, Hk, dk, dv, parts)
   if (DKP == 64) {
     if (DVP == 64) LAUNCH_M(64, 64);
     else if (DVP == 128) LAUNCH_M(64, 128);

@@ -45,18 +45,19 @@ void mix_scalar_rmsnorm(void*, const float*, const float*, float, long, int,
                         int, hipStream_t);
 void mix_attn_prep(void*, const void*, long, int, int, int, const float*,
                    const float*, float, const float*, int, const long*, void*,
-                   void*, long, int, int, int, int, int, int, hipStream_t);
+                   void*, const void*, long, const float*, long, int, int, int,
+                   int, int, int, hipStream_t);
 void mix_local_attention(void*, long, int, const void*, const void*,
                          const void*, const int*, int, const int*, const int*,
                          const int*, float, int, int, const void*, long, int,
-                         float, const float*, const float*, int, long, long,
-                         int, int, int, int, int, int, hipStream_t);
+                         float, const float*, const float*, int, int, long,
+                         long, int, int, int, int, int, int, hipStream_t);
 int mix_local_attention_mfma(void*, long, int, const void*, const void*,
                              const void*, const int*, int, const int*,
                              const int*, const int*, const int*, int, float,
                              int, int, const void*, long, int, float,
                              const float*, const float*, int, int, int, int,
-                             int, int, hipStream_t);
+                             int, int, int, hipStream_t);
 void mix_token_embed(float*, const long*, const long*, const long*,
                      const void*, const void*, long, long, long, const float*,
                      float, long, int, int, hipStream_t);
@@ -70,7 +71,31 @@ void mix_moe_dispatch(int*, int*, int*, int*, const int*, long, int, int, int,
                       long, hipStream_t);
 void mix_expert_gemm_plain(void*, const void*, const void*, const int*,
                            const int*, const int*, int, int, int, int, long,
-                           int, int, hipStream_t);
+                           int, float, int, hipStream_t);
+void sutro_grouped_gemm_glu(void*, const void*, const void*, const int*,
+                            const int*, const int*, int, int, int, long, int,
+                            float, hipStream_t);
+void mix_add_rmsnorm(float*, const void*, const void*, const int*,
+                     const float*, int, const float*, const void*, const void*,
+                     const void*, long, int, const float*, float, void*, long,
+                     int, int, hipStream_t);
+void mix_glu_mul(void*, const void*, long, int, int, long, int, int, float,
+                 int, hipStream_t);
+void mix_moe_route_softmax(int*, float*, float*, const float*, const float*,
+                           long, int, int, int, int, int, float, hipStream_t);
+void mix_silu_sections(float*, const void*, long, int, int, int, int, int, int,
+                       long, int, hipStream_t);
+void mix_gated_group_norm(void*, long, int, const float*, const void*, long,
+                          int, const float*, float, long, int, int, int, int,
+                          hipStream_t);
+void mix_ssd_prep(float*, float*, float*, const void*, long, int, int,
+                  const float*, const float*, int, const float*, const float*,
+                  float*, const int*, const int*, const int*, const int*, long,
+                  int, int, int, int, hipStream_t);
+int mix_decay_scan(float*, const float*, long, const float*, long,
+                   const float*, long, const float*, long, const float*,
+                   const float*, float*, const int*, const int*, const int*,
+                   int, int, int, int, int, hipStream_t);
 void mix_softcap(float*, const void*, float, long, int, hipStream_t);
 void sutro_grouped_gemm(void*, const void*, const void*, const int*,
                         const int*, const int*, int, int, int, long, int,
@@ -163,7 +188,8 @@ void attn_prep(torch::Tensor q_out, torch::Tensor proj, long q_off, long k_off,
                c10::optional<torch::Tensor> k_w, double eps,
                torch::Tensor cos_sin, torch::Tensor slots,
                torch::Tensor k_cache,
-               torch::Tensor v_cache) {
+               torch::Tensor v_cache, c10::optional<torch::Tensor> v_first,
+               long v_first_off, c10::optional<torch::Tensor> v_lambda) {
   CHECK_GPU(proj); CHECK_GPU(q_out); CHECK_CONTIG(q_out);
   CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
   CHECK_I64(slots); CHECK_F32(cos_sin); CHECK_CONTIG(cos_sin);
@@ -194,10 +220,26 @@ void attn_prep(torch::Tensor q_out, torch::Tensor proj, long q_off, long k_off,
     CHECK_F32(*k_w); TORCH_CHECK(k_w->numel() == dk, "k norm size");
     kw = k_w->data_ptr<float>();
   }
+  // values blended with another layer's values of the same tokens
+  const void* vf = nullptr; long ldvf = 0; const float* vl = nullptr;
+  if (v_first.has_value()) {
+    TORCH_CHECK(v_lambda.has_value(), "value blending needs its weight");
+    CHECK_GPU(*v_first); CHECK_GPU(*v_lambda); CHECK_F32(*v_lambda);
+    TORCH_CHECK(v_first->scalar_type() == proj.scalar_type() &&
+                v_first->dim() == 2 && v_first->size(0) == T &&
+                v_first->stride(1) == 1 && v_lambda->numel() == 1,
+                "blended values: dtype or rows");
+    check_proj(*v_first, v_first_off, G * dv, "first values");
+    vf = (const char*)v_first->data_ptr() +
+         v_first_off * (long)v_first->element_size();
+    ldvf = v_first->stride(0);
+    vl = v_lambda->data_ptr<float>();
+  }
   mix_attn_prep(q_out.data_ptr(), proj.data_ptr(), proj.stride(0), (int)q_off,
                 (int)k_off, (int)v_off, qw, kw, (float)eps,
                 cos_sin.data_ptr<float>(), (int)half, slots.data_ptr<long>(),
-                k_cache.data_ptr(), v_cache.data_ptr(), T, (int)H, (int)G,
+                k_cache.data_ptr(), v_cache.data_ptr(), vf, ldvf, vl, T,
+                (int)H, (int)G,
                 (int)dk, (int)dv, (int)page, act_kind(proj), cur_stream());
 }
 
@@ -210,7 +252,8 @@ void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
                      c10::optional<torch::Tensor> tile_seq,
                      c10::optional<torch::Tensor> tile_q0,
                      long prefill_rows, c10::optional<torch::Tensor> bias_r1,
-                     c10::optional<torch::Tensor> bias_r2, bool sink) {
+                     c10::optional<torch::Tensor> bias_r2, bool sink,
+                     long keep_first) {
   CHECK_GPU(q); CHECK_CONTIG(q); CHECK_CONTIG(k_cache); CHECK_CONTIG(v_cache);
   CHECK_I32(bt); CHECK_I32(seq_lens); CHECK_I32(qlocs); CHECK_I32(token_seq);
   CHECK_CONTIG(bt);
@@ -255,8 +298,8 @@ void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
             tile_seq->data_ptr<int>(), tile_q0->data_ptr<int>(),
             (int)tile_seq->numel(), (float)scale, (int)chunk, (int)window,
             proj.data_ptr(), proj.stride(0), (int)gate_off, (float)out_scale,
-            r1, r2, sink ? 1 : 0, (int)H, (int)G, (int)dk, (int)dv, (int)page,
-            cur_stream()))
+            r1, r2, sink ? 1 : 0, (int)keep_first, (int)H, (int)G, (int)dk,
+            (int)dv, (int)page, cur_stream()))
       t0 = prefill_rows;
   }
   if (t0 < T)
@@ -267,7 +310,7 @@ void local_attention(torch::Tensor out, long out_off, torch::Tensor q,
                         token_seq.data_ptr<int>(), (float)scale, (int)chunk,
                         (int)window, proj.data_ptr(), proj.stride(0),
                         (int)gate_off, (float)out_scale, r1, r2, sink ? 1 : 0,
-                        t0, T - t0, (int)H,
+                        (int)keep_first, t0, T - t0, (int)H,
                         (int)G, (int)dk, (int)dv, (int)page, act_kind(q),
                         cur_stream());
 }
@@ -730,15 +773,21 @@ void moe_dispatch(torch::Tensor row_tok, torch::Tensor tile_off,
 
 void expert_gemm(torch::Tensor out, torch::Tensor a, torch::Tensor w,
                  c10::optional<torch::Tensor> row_tok, torch::Tensor tile_off,
-                 torch::Tensor counts, long act, long bm) {
+                 torch::Tensor counts, long act, long bm, double limit) {
   CHECK_GPU(a); CHECK_CONTIG(a); CHECK_GPU(w); CHECK_CONTIG(w);
   CHECK_GPU(out); CHECK_CONTIG(out);
   CHECK_I32(tile_off); CHECK_I32(counts); CHECK_GPU(tile_off); CHECK_GPU(counts);
+  CHECK_CONTIG(tile_off); CHECK_CONTIG(counts);
   TORCH_CHECK(w.dim() == 3 && a.dim() == 2 && out.dim() == 2, "operand ranks");
-  const long E = w.size(0), N = w.size(1), K = w.size(2);
+  const bool glu = act == 3;   // w rows: gate rows, then up rows
+  const long E = w.size(0), K = w.size(2);
+  const long N = glu ? w.size(1) / 2 : w.size(1);
   const long n_rows = out.size(0);
   TORCH_CHECK(bm == 64 || bm == 128, "bm must be 64 or 128");
-  TORCH_CHECK(act == 0 || act == 2, "activation: 0 (none) or 2 (relu squared)");
+  TORCH_CHECK(act == 0 || act == 2 || act == 3,
+              "activation: 0 (none), 2 (relu squared) or 3 (clamped unit)");
+  TORCH_CHECK(!glu || (w.size(1) % 2 == 0 && limit > 0),
+              "the clamped unit needs gate and up rows and a limit");
   TORCH_CHECK(a.size(1) == K && out.size(1) == N && n_rows % bm == 0 &&
               counts.numel() == E && tile_off.numel() == E + 1,
               "operand shapes");
@@ -752,19 +801,278 @@ void expert_gemm(torch::Tensor out, torch::Tensor a, torch::Tensor w,
   } else {
     TORCH_CHECK(a.size(0) == n_rows, "a must be laid out in segments");
   }
-  TORCH_CHECK((act == 2) == (rt != nullptr),
+  TORCH_CHECK((act != 0) == (rt != nullptr),
               "the gathered stage carries the activation");
   if (kind == 0 && K % 64 == 0 && N % 64 == 0) {
-    sutro_grouped_gemm(out.data_ptr(), a.data_ptr(), w.data_ptr(), rt,
-                       tile_off.data_ptr<int>(), counts.data_ptr<int>(), (int)E,
-                       (int)(n_rows / bm), (int)N, K, (int)act, (int)bm,
-                       cur_stream());
+    if (glu)
+      sutro_grouped_gemm_glu(out.data_ptr(), a.data_ptr(), w.data_ptr(), rt,
+                             tile_off.data_ptr<int>(), counts.data_ptr<int>(),
+                             (int)E, (int)(n_rows / bm), (int)N, K, (int)bm,
+                             (float)limit, cur_stream());
+    else
+      sutro_grouped_gemm(out.data_ptr(), a.data_ptr(), w.data_ptr(), rt,
+                         tile_off.data_ptr<int>(), counts.data_ptr<int>(),
+                         (int)E, (int)(n_rows / bm), (int)N, K, (int)act,
+                         (int)bm, cur_stream());
     return;
   }
   mix_expert_gemm_plain(out.data_ptr(), a.data_ptr(), w.data_ptr(), rt,
                         tile_off.data_ptr<int>(), counts.data_ptr<int>(),
                         (int)E, (int)N, (int)K, (int)bm, n_rows,
-                        act == 2 ? 1 : 0, kind, cur_stream());
+                        act == 2 ? 1 : (glu ? 2 : 0), (float)limit, kind,
+                        cur_stream());
+}
+
+// ---- pre-norm layers, decay recurrences ----
+
+static const void* opt_ptr(const c10::optional<torch::Tensor>& t) {
+  return t.has_value() ? t->data_ptr() : nullptr;
+}
+
+void add_rmsnorm(torch::Tensor x, c10::optional<torch::Tensor> y,
+                 c10::optional<torch::Tensor> rows,
+                 c10::optional<torch::Tensor> padpos,
+                 c10::optional<torch::Tensor> wts,
+                 c10::optional<torch::Tensor> idw,
+                 c10::optional<torch::Tensor> h_in,
+                 c10::optional<torch::Tensor> y2,
+                 c10::optional<torch::Tensor> proj2, long sg_off,
+                 c10::optional<torch::Tensor> norm_w, double eps,
+                 c10::optional<torch::Tensor> h_out) {
+  CHECK_GPU(x); CHECK_CONTIG(x); CHECK_F32(x);
+  TORCH_CHECK(x.dim() == 2, "x must be [T, W]");
+  const long T = x.size(0), W = x.size(1);
+  int kind = -1;
+  auto act = [&](const torch::Tensor& t, const char* what) {
+    CHECK_GPU(t); CHECK_CONTIG(t);
+    const int k = act_kind(t);
+    TORCH_CHECK(kind < 0 || kind == k, what, ": activation dtypes differ");
+    kind = k;
+  };
+  auto rowsok = [&](const torch::Tensor& t, const char* what) {
+    act(t, what);
+    TORCH_CHECK(t.dim() == 2 && t.size(0) == T && t.size(1) == W, what,
+                " must be [T, W]");
+  };
+  if (y.has_value()) rowsok(*y, "y");
+  if (y2.has_value()) rowsok(*y2, "y2");
+  if (h_in.has_value()) rowsok(*h_in, "h_in");
+  if (h_out.has_value()) {
+    rowsok(*h_out, "h_out");
+    TORCH_CHECK(norm_w.has_value(), "a normed output needs the norm weight");
+    CHECK_GPU(*norm_w); CHECK_F32(*norm_w); CHECK_CONTIG(*norm_w);
+    TORCH_CHECK(norm_w->numel() == W, "norm weight size");
+  }
+  int k = 0;
+  if (rows.has_value()) {
+    act(*rows, "rows");
+    TORCH_CHECK(padpos.has_value() && wts.has_value(),
+                "expert rows need padpos and weights");
+    CHECK_GPU(*padpos); CHECK_I32(*padpos); CHECK_CONTIG(*padpos);
+    CHECK_GPU(*wts); CHECK_F32(*wts); CHECK_CONTIG(*wts);
+    TORCH_CHECK(rows->dim() == 2 && rows->size(1) == W && padpos->dim() == 2 &&
+                padpos->size(0) == T && wts->sizes() == padpos->sizes(),
+                "expert rows / padpos / weights shapes");
+    k = (int)padpos->size(1);
+  }
+  if (idw.has_value()) {
+    CHECK_GPU(*idw); CHECK_F32(*idw); CHECK_CONTIG(*idw);
+    TORCH_CHECK(idw->numel() == T && h_in.has_value(),
+                "identity weights need one number a token and the input");
+  }
+  long ld2 = 0;
+  if (y2.has_value() && sg_off >= 0) {
+    TORCH_CHECK(proj2.has_value(), "the gate of y2 needs its projection");
+    CHECK_GPU(*proj2);
+    TORCH_CHECK(act_kind(*proj2) == kind && proj2->size(0) == T,
+                "gate projection dtype or rows");
+    check_proj(*proj2, sg_off, 1, "shared gate");
+    ld2 = proj2->stride(0);
+  }
+  if (kind < 0) kind = 1;
+  mix_add_rmsnorm(x.data_ptr<float>(), opt_ptr(y), opt_ptr(rows),
+                  (const int*)opt_ptr(padpos), (const float*)opt_ptr(wts), k,
+                  idw.has_value() ? (const float*)opt_ptr(idw) : nullptr,
+                  idw.has_value() ? opt_ptr(h_in) : nullptr, opt_ptr(y2),
+                  (y2.has_value() && sg_off >= 0) ? opt_ptr(proj2) : nullptr,
+                  ld2, (int)sg_off, (const float*)opt_ptr(norm_w), (float)eps,
+                  h_out.has_value() ? h_out->data_ptr() : nullptr, T, (int)W,
+                  kind, cur_stream());
+}
+
+void glu_mul(torch::Tensor out, torch::Tensor proj, long gate_off, long up_off,
+             long act, double limit) {
+  CHECK_GPU(proj); CHECK_GPU(out); CHECK_CONTIG(out);
+  const long T = out.size(0), F = out.size(1);
+  TORCH_CHECK(out.scalar_type() == proj.scalar_type(), "dtype mismatch");
+  TORCH_CHECK(act >= 0 && act <= 2 && (act != 2 || limit > 0),
+              "unit: 0 tanh-GELU, 1 silu, 2 clamped (with a limit)");
+  check_proj(proj, gate_off, F, "gate");
+  check_proj(proj, up_off, F, "up");
+  TORCH_CHECK(proj.size(0) == T, "row mismatch");
+  mix_glu_mul(out.data_ptr(), proj.data_ptr(), proj.stride(0), (int)gate_off,
+              (int)up_off, T, (int)F, (int)act, (float)limit, act_kind(proj),
+              cur_stream());
+}
+
+void moe_route_softmax(torch::Tensor idx, torch::Tensor wts, torch::Tensor idw,
+                       torch::Tensor logits, c10::optional<torch::Tensor> corr,
+                       long groups, long keep, long n_real, double scale) {
+  CHECK_GPU(logits); CHECK_F32(logits); CHECK_CONTIG(logits);
+  CHECK_GPU(idx); CHECK_I32(idx); CHECK_CONTIG(idx);
+  CHECK_GPU(wts); CHECK_F32(wts); CHECK_CONTIG(wts);
+  CHECK_GPU(idw); CHECK_F32(idw); CHECK_CONTIG(idw);
+  TORCH_CHECK(logits.dim() == 2 && idx.dim() == 2, "operand ranks");
+  const long T = logits.size(0), n = logits.size(1), top = idx.size(1);
+  TORCH_CHECK(idx.size(0) == T && wts.sizes() == idx.sizes() &&
+              idw.numel() == T, "output shapes");
+  TORCH_CHECK(groups >= 1 && groups <= 1024 && n % groups == 0 && keep >= 1 &&
+              keep <= groups && top >= 1 && top <= keep * (n / groups) &&
+              n_real >= 0 && n_real <= n && n <= 4096,
+              "router shape: groups, kept groups or choices");
+  const float* cp = nullptr;
+  if (corr.has_value()) {
+    CHECK_GPU(*corr); CHECK_F32(*corr); CHECK_CONTIG(*corr);
+    TORCH_CHECK(corr->numel() == n, "one correction per router output");
+    cp = corr->data_ptr<float>();
+  }
+  mix_moe_route_softmax(idx.data_ptr<int>(), wts.data_ptr<float>(),
+                        idw.data_ptr<float>(), logits.data_ptr<float>(), cp, T,
+                        (int)n, (int)n_real, (int)top, (int)groups, (int)keep,
+                        (float)scale, cur_stream());
+}
+
+void silu_sections(torch::Tensor out, torch::Tensor proj,
+                   std::vector<long> offs, std::vector<long> sizes) {
+  CHECK_GPU(proj); CHECK_GPU(out); CHECK_F32(out); CHECK_CONTIG(out);
+  TORCH_CHECK(offs.size() == sizes.size() && offs.size() >= 1 &&
+              offs.size() <= 3, "one to three sections");
+  long o[3] = {0, 0, 0}, n[3] = {0, 0, 0}, tot = 0;
+  for (size_t i = 0; i < offs.size(); ++i) {
+    check_proj(proj, offs[i], sizes[i], "section");
+    o[i] = offs[i]; n[i] = sizes[i]; tot += sizes[i];
+  }
+  const long T = proj.size(0);
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == tot,
+              "output shape");
+  mix_silu_sections(out.data_ptr<float>(), proj.data_ptr(), proj.stride(0),
+                    (int)o[0], (int)n[0], (int)o[1], (int)n[1], (int)o[2],
+                    (int)n[2], T, act_kind(proj), cur_stream());
+}
+
+void gated_group_norm(torch::Tensor out, long out_off, torch::Tensor o,
+                      torch::Tensor proj, long g_off, torch::Tensor norm_w,
+                      double eps, long groups, bool gate_first) {
+  CHECK_GPU(o); CHECK_F32(o); CHECK_CONTIG(o); CHECK_GPU(proj); CHECK_GPU(out);
+  CHECK_GPU(norm_w); CHECK_F32(norm_w); CHECK_CONTIG(norm_w);
+  const long T = o.size(0);
+  const long n = T ? o.numel() / T : norm_w.numel();
+  TORCH_CHECK(norm_w.numel() == n && groups >= 1 && n % groups == 0,
+              "norm weight size or parts");
+  TORCH_CHECK(out.dim() == 2 && out.stride(1) == 1 && out.size(0) == T &&
+              out_off >= 0 && out_off + n <= out.size(1), "out section");
+  TORCH_CHECK(out.scalar_type() == proj.scalar_type() && proj.size(0) == T,
+              "dtype or rows");
+  check_proj(proj, g_off, n, "gate");
+  mix_gated_group_norm(out.data_ptr(), out.stride(0), (int)out_off,
+                       o.data_ptr<float>(), proj.data_ptr(), proj.stride(0),
+                       (int)g_off, norm_w.data_ptr<float>(), (float)eps, T,
+                       (int)n, (int)groups, gate_first ? 1 : 0, act_kind(proj),
+                       cur_stream());
+}
+
+void ssd_prep(torch::Tensor xbc, torch::Tensor decay, torch::Tensor dt,
+              torch::Tensor proj, long xbc_off, long dt_off,
+              torch::Tensor conv_wt, torch::Tensor conv_b,
+              torch::Tensor dt_bias, torch::Tensor a_log,
+              torch::Tensor conv_state, torch::Tensor state_slots,
+              torch::Tensor qlocs, torch::Tensor seq_lens,
+              torch::Tensor token_seq) {
+  CHECK_GPU(proj); CHECK_GPU(xbc); CHECK_F32(xbc); CHECK_CONTIG(xbc);
+  CHECK_F32(decay); CHECK_CONTIG(decay); CHECK_F32(dt); CHECK_CONTIG(dt);
+  CHECK_GPU(conv_wt); CHECK_F32(conv_wt); CHECK_CONTIG(conv_wt);
+  CHECK_GPU(conv_b); CHECK_F32(conv_b); CHECK_CONTIG(conv_b);
+  CHECK_GPU(dt_bias); CHECK_F32(dt_bias); CHECK_GPU(a_log); CHECK_F32(a_log);
+  CHECK_GPU(conv_state); CHECK_F32(conv_state); CHECK_CONTIG(conv_state);
+  CHECK_I32(state_slots); CHECK_I32(qlocs); CHECK_I32(seq_lens);
+  CHECK_I32(token_seq);
+  const long T = proj.size(0), C = xbc.size(1), H = decay.size(1);
+  const long taps = conv_wt.size(0), S = seq_lens.numel();
+  TORCH_CHECK(xbc.size(0) == T && decay.size(0) == T && dt.sizes() ==
+              decay.sizes() && conv_wt.dim() == 2 && conv_wt.size(1) == C &&
+              conv_b.numel() == C && dt_bias.numel() == H &&
+              a_log.numel() == H, "operand shapes");
+  TORCH_CHECK(conv_state.dim() == 3 && conv_state.size(2) == C &&
+              conv_state.size(1) == std::max<long>(1, taps - 1),
+              "filter history shape");
+  TORCH_CHECK(token_seq.numel() == T && qlocs.numel() == S + 1 &&
+              state_slots.numel() == S, "batch metadata sizes");
+  check_proj(proj, xbc_off, C, "x|B|C");
+  check_proj(proj, dt_off, H, "dt");
+  mix_ssd_prep(xbc.data_ptr<float>(), decay.data_ptr<float>(),
+               dt.data_ptr<float>(), proj.data_ptr(), proj.stride(0),
+               (int)xbc_off, (int)dt_off, conv_wt.data_ptr<float>(),
+               conv_b.data_ptr<float>(), (int)taps, dt_bias.data_ptr<float>(),
+               a_log.data_ptr<float>(), conv_state.data_ptr<float>(),
+               state_slots.data_ptr<int>(), qlocs.data_ptr<int>(),
+               seq_lens.data_ptr<int>(), token_seq.data_ptr<int>(), T, (int)S,
+               (int)C, (int)H, act_kind(proj), cur_stream());
+}
+
+void decay_scan(torch::Tensor o, torch::Tensor q, torch::Tensor k,
+                torch::Tensor v, torch::Tensor decay,
+                c10::optional<torch::Tensor> gain,
+                c10::optional<torch::Tensor> skip, torch::Tensor state,
+                torch::Tensor state_slots, torch::Tensor qlocs,
+                torch::Tensor seq_lens) {
+  CHECK_GPU(o); CHECK_F32(o); CHECK_CONTIG(o);
+  CHECK_GPU(q); CHECK_F32(q); CHECK_GPU(k); CHECK_F32(k);
+  CHECK_GPU(v); CHECK_F32(v); CHECK_GPU(decay); CHECK_F32(decay);
+  CHECK_CONTIG(decay);
+  CHECK_GPU(state); CHECK_F32(state); CHECK_CONTIG(state);
+  CHECK_I32(state_slots); CHECK_I32(qlocs); CHECK_I32(seq_lens);
+  TORCH_CHECK(q.dim() == 3 && k.dim() == 3 && v.dim() == 3, "q, k, v ranks");
+  const long T = v.size(0), H = v.size(1), dv = v.size(2);
+  const long G = k.size(1), dk = k.size(2), S = seq_lens.numel();
+  // rows may be strided (views of one buffer); heads and channels are dense
+  auto dense = [](const torch::Tensor& t) {
+    return t.stride(2) == 1 && t.stride(1) == t.size(2);
+  };
+  TORCH_CHECK(dense(q) && dense(k) && dense(v), "heads must be dense");
+  TORCH_CHECK(q.sizes() == k.sizes() && q.size(0) == T && H % G == 0 &&
+              o.size(0) == T && o.size(1) == H && o.size(2) == dv,
+              "q / k / v / o shapes");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == dk &&
+              state.size(3) == dv, "state shape");
+  TORCH_CHECK(qlocs.numel() == S + 1 && state_slots.numel() == S,
+              "batch metadata sizes");
+  long lda = 0;
+  if (decay.dim() == 2) {
+    TORCH_CHECK(decay.size(0) == T && decay.size(1) == H, "decay shape");
+    lda = H;
+  } else {
+    TORCH_CHECK(decay.dim() == 1 && decay.numel() == H, "decay shape");
+  }
+  const float* gp = nullptr; const float* sp = nullptr;
+  if (gain.has_value()) {
+    CHECK_GPU(*gain); CHECK_F32(*gain); CHECK_CONTIG(*gain);
+    TORCH_CHECK(gain->numel() == T * H, "gain shape");
+    gp = gain->data_ptr<float>();
+  }
+  if (skip.has_value()) {
+    CHECK_GPU(*skip); CHECK_F32(*skip); CHECK_CONTIG(*skip);
+    TORCH_CHECK(skip->numel() == H, "skip shape");
+    sp = skip->data_ptr<float>();
+  }
+  if (T == 0) return;
+  const int ok = mix_decay_scan(
+      o.data_ptr<float>(), q.data_ptr<float>(), q.stride(0),
+      k.data_ptr<float>(), k.stride(0), v.data_ptr<float>(), v.stride(0),
+      decay.data_ptr<float>(), lda, gp, sp, state.data_ptr<float>(),
+      state_slots.data_ptr<int>(), qlocs.data_ptr<int>(),
+      seq_lens.data_ptr<int>(), (int)S, (int)H, (int)G, (int)dk, (int)dv,
+      cur_stream());
+  TORCH_CHECK(ok, "decay_scan: key size above 256 is unsupported");
 }
 
 void softcap(torch::Tensor out, torch::Tensor z, double cap) {
@@ -776,11 +1084,27 @@ void softcap(torch::Tensor out, torch::Tensor z, double cap) {
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("add_rmsnorm", &add_rmsnorm,
+        "x += y + expert rows + identity share + gated y2; h = rmsnorm(x) * w");
+  m.def("glu_mul", &glu_mul, "act(gate) * up: tanh-GELU, silu or clamped unit");
+  m.def("moe_route_softmax", &moe_route_softmax,
+        "softmax router: correction, group-limited choice, identity experts");
+  m.def("silu_sections", &silu_sections, "fp32 silu of projection sections");
+  m.def("gated_group_norm", &gated_group_norm,
+        "gated read-out normed in equal parts");
+  m.def("ssd_prep", &ssd_prep, "Mamba-2 inputs: filter, silu, step, decay");
+  m.def("decay_scan", &decay_scan, "S <- a S + b k v^T; o = S^T q + skip v");
   m.def("gelu_tanh_mul", &gelu_tanh_mul, "tanh-GELU(gate) * up");
   m.def("gated_norm_residual", &gated_norm_residual,
         "x += m * g * n(y * sigmoid(gate)); h = cast(x)");
   m.def("scalar_rmsnorm", &scalar_rmsnorm, "RMS norm with one scalar gain");
-  m.def("attn_prep", &attn_prep, "q/k norm + partial rotation + paged K/V write");
+  m.def("attn_prep", &attn_prep,
+        "q/k norm + partial rotation + value blending + paged K/V write",
+        py::arg("q"), py::arg("proj"), py::arg("q_off"), py::arg("k_off"),
+        py::arg("v_off"), py::arg("q_w"), py::arg("k_w"), py::arg("eps"),
+        py::arg("cos_sin"), py::arg("slots"), py::arg("k_cache"),
+        py::arg("v_cache"), py::arg("v_first") = c10::nullopt,
+        py::arg("v_first_off") = 0, py::arg("v_lambda") = c10::nullopt);
   m.def("local_attention", &local_attention,
         "chunked/windowed paged attention with per-head output gate",
         py::arg("out"), py::arg("out_off"), py::arg("q"), py::arg("k_cache"),
@@ -790,7 +1114,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("gate_off"), py::arg("out_scale"),
         py::arg("tile_seq") = c10::nullopt, py::arg("tile_q0") = c10::nullopt,
         py::arg("prefill_rows") = 0, py::arg("bias_r1") = c10::nullopt,
-        py::arg("bias_r2") = c10::nullopt, py::arg("sink") = false);
+        py::arg("bias_r2") = c10::nullopt, py::arg("sink") = false,
+        py::arg("keep_first") = 0);
   m.def("delta_prep", &delta_prep, "delta-rule inputs: filters, norms, gates",
         py::arg("qn"), py::arg("kn"), py::arg("v"), py::arg("decay"),
         py::arg("beta"), py::arg("proj"), py::arg("q_off"), py::arg("k_off"),
@@ -827,6 +1152,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "(token, choice) pairs -> padded per-expert segments");
   m.def("expert_gemm", &expert_gemm,
         "GEMM over padded per-expert segments (matrix cores for bf16 with "
-        "64-aligned sizes, plain tiles otherwise)");
+        "64-aligned sizes, plain tiles otherwise)",
+        py::arg("out"), py::arg("a"), py::arg("w"), py::arg("row_tok"),
+        py::arg("tile_off"), py::arg("counts"), py::arg("act"), py::arg("bm"),
+        py::arg("limit") = 0.0);
   m.def("softcap", &softcap, "cap * tanh(z / cap), fp32 out");
 }

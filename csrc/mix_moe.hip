@@ -258,13 +258,18 @@ extern "C" void mix_moe_dispatch(int* row_tok, int* tile_off, int* counts,
 // out[r, n] = act(sum_k a[tok(r), k] * w[e, n, k]) over 64-row tiles of the
 // padded segments; 256 threads as 16 x 16, 4 x 4 outputs a thread, K staged
 // 16 at a time through LDS. Rows past a segment's live count are not stored.
+// act 1: relu(x)^2. act 2: w holds N gate rows then N up rows per expert and
+// out[r, n] = g sigmoid(1.702 g) (u + 1), g = min(gate, limit), u = clamp(up).
 template <typename A>
 __global__ void __launch_bounds__(256) expert_gemm_plain_kernel(
     A* __restrict__ out, const A* __restrict__ a, const A* __restrict__ w,
     const int* __restrict__ row_tok, const int* __restrict__ tile_off,
-    const int* __restrict__ counts, int E, int N, int K, int bm, int relu2) {
+    const int* __restrict__ counts, int E, int N, int K, int bm, int act,
+    float limit) {
   __shared__ float As[16][65];
   __shared__ float Bs[16][65];
+  __shared__ float Us[16][65];
+  const bool glu = act == 2;
   const int tiles_per = bm / 64;
   const int t64 = blockIdx.x;              // 64-row tile over all segments
   const int t = t64 / tiles_per;           // bm-row tile
@@ -280,14 +285,14 @@ __global__ void __launch_bounds__(256) expert_gemm_plain_kernel(
   if (live <= 0) return;
   const long seg = (long)tile_off[e] * bm + m0;
   const int n0 = blockIdx.y * 64;
-  const A* we = w + (long)e * N * K;
+  const A* we = w + (long)e * (glu ? 2 : 1) * N * K;
   const int tid = threadIdx.x;
   const int tx = tid & 15, ty = tid >> 4;
-  float acc[4][4];
+  float acc[4][4], accu[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) acc[i][j] = accu[i][j] = 0.f;
   // staging: thread -> (row = tid / 4, 4 consecutive k)
   const int sr = tid >> 2, sk = (tid & 3) * 4;
   long arow = -1;
@@ -299,6 +304,9 @@ __global__ void __launch_bounds__(256) expert_gemm_plain_kernel(
       const int kk = k0 + sk + q;
       As[sk + q][sr] = (arow >= 0 && kk < K) ? ldf<A>(a + arow * K + kk) : 0.f;
       Bs[sk + q][sr] = (bn < N && kk < K) ? ldf<A>(we + (long)bn * K + kk) : 0.f;
+      if (glu)
+        Us[sk + q][sr] =
+            (bn < N && kk < K) ? ldf<A>(we + (long)(N + bn) * K + kk) : 0.f;
     }
     __syncthreads();
 #pragma unroll
@@ -312,6 +320,14 @@ __global__ void __launch_bounds__(256) expert_gemm_plain_kernel(
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] += av[i] * bv[j];
+      if (glu) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bv[j] = Us[kk][tx * 4 + j];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) accu[i][j] += av[i] * bv[j];
+      }
     }
     __syncthreads();
   }
@@ -324,9 +340,13 @@ __global__ void __launch_bounds__(256) expert_gemm_plain_kernel(
       const int n = n0 + tx * 4 + j;
       if (n >= N) continue;
       float v = acc[i][j];
-      if (relu2) {
+      if (act == 1) {
         v = v > 0.f ? v : 0.f;
         v *= v;
+      } else if (glu) {
+        const float g = fminf(v, limit);
+        const float u = fminf(fmaxf(accu[i][j], -limit), limit);
+        v = g * sigmoid_f(1.702f * g) * (u + 1.f);
       }
       stf<A>(out + (seg + r) * N + n, v);
     }
@@ -336,19 +356,19 @@ __global__ void __launch_bounds__(256) expert_gemm_plain_kernel(
 extern "C" void mix_expert_gemm_plain(void* out, const void* a, const void* w,
                                       const int* row_tok, const int* tile_off,
                                       const int* counts, int E, int N, int K,
-                                      int bm, long n_rows, int relu2, int f32,
-                                      hipStream_t s) {
+                                      int bm, long n_rows, int act, float limit,
+                                      int f32, hipStream_t s) {
   const long tiles = n_rows / 64;
   if (tiles == 0) return;
   const dim3 grid((unsigned)tiles, (unsigned)((N + 63) / 64));
   if (f32)
     hipLaunchKernelGGL(expert_gemm_plain_kernel<float>, grid, dim3(256), 0, s,
                        (float*)out, (const float*)a, (const float*)w, row_tok,
-                       tile_off, counts, E, N, K, bm, relu2);
+                       tile_off, counts, E, N, K, bm, act, limit);
   else
     hipLaunchKernelGGL(expert_gemm_plain_kernel<u16>, grid, dim3(256), 0, s,
                        (u16*)out, (const u16*)a, (const u16*)w, row_tok,
-                       tile_off, counts, E, N, K, bm, relu2);
+                       tile_off, counts, E, N, K, bm, act, limit);
 }
 
 // ---- softcap ---------------------------------------------------------------

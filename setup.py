@@ -38,6 +38,8 @@ MIX_SOURCES = [
     "csrc/mix_prep.hip",
     "csrc/mix_mlstm.hip",
     "csrc/mix_moe.hip",
+    "csrc/mix_prenorm.hip",
+    "csrc/mix_decay.hip",
     # the matrix-core expert GEMM serves both extensions
     "csrc/grouped_gemm.hip",
 ]

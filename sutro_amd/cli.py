@@ -217,7 +217,8 @@ def generate(model: str, prompts, max_tokens: int, temperature: float,
     if cfg.device.startswith("cuda"):
         from .build import ensure_built
 
-        layer_list = cfg.spec.arch in ("vodinex", "ruludra", "vukotar")
+        layer_list = cfg.spec.arch in ("vodinex", "ruludra", "vukotar",
+                                      "nosalorn")
         ensure_built(["_C", "_C_mix"] if layer_list else ["_C"])
     eng = LLMEngine(cfg)
     outs = eng.generate(list(prompts), sampling=SamplingParams(

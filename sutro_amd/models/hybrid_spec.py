@@ -3,7 +3,7 @@ mixer and feed-forward, so attention layers, recurrent layers and layers that
 run both side by side can be ordered freely.
 
 A spec is built from a checkpoint's ``config.json`` (see :func:`vodinex_spec`,
-:func:`ruludra_spec` and :func:`vukotar_spec`)
+:func:`ruludra_spec`, :func:`vukotar_spec` and :func:`nosalorn_spec`)
 or directly in code (tests, benchmarks). Nothing here fixes a size: widths,
 head counts, mask sizes, filter lengths and the order of layers all come from
 the config.
@@ -22,8 +22,18 @@ class AttnMixerSpec:
     ``chunk``: a query at position i sees keys j <= i with
     ``j // chunk == i // chunk`` (0 = no chunking). ``window``: a query sees
     at most the last ``window`` keys (0 = unlimited). Both may be combined.
+    ``keep_first``: with a window, keys at positions below `keep_first` stay
+    visible to every later query (at their true positions).
     ``rot_dims``: how many leading dimensions of each head are rotated
-    (rotate-half pairing inside that prefix); 0 = no rotation."""
+    (rotate-half pairing inside that prefix); 0 = no rotation.
+    ``rot_scaling``: (factor, original length, fast turns, slow turns) of a
+    YaRN frequency blend: frequencies that turn fewer than `slow` times over
+    the original length are divided by `factor`, those that turn more than
+    `fast` times are kept, a linear ramp over the pair index lies between,
+    and cos / sin are multiplied by 0.1 ln(factor) + 1.
+    ``v_mix``: the values of every such layer but the first are blended with
+    the first such layer's values of the same token, v <- (1 - l) v + l v1,
+    with a learned scalar l; the blend is what the cache holds."""
 
     heads: int
     kv_heads: int
@@ -40,6 +50,10 @@ class AttnMixerSpec:
     # a silent sink: a key of score 0 without a value takes part in the
     # normalisation, p_j = exp(s_j) / (1 + sum_j exp(s_j))
     sink: bool = False
+    keep_first: int = 0
+    rot_scaling: Optional[Tuple[float, float, float, float]] = None
+    v_mix: bool = False
+    out_bias: bool = True    # with `bias`: the output projection has one too
 
 
 @dataclass(frozen=True)
@@ -120,8 +134,38 @@ class MLSTMMixerSpec:
     gate_cap: float
 
 
+@dataclass(frozen=True)
+class DecayAttnMixerSpec:
+    """Linear attention with one fixed decay per head ("lightning"
+    attention): q, k, v pass silu, S_t = decay_h S_(t-1) + k_t v_t^T,
+    o_t = S_t^T q_t; the concatenated heads pass one RMS norm (weighted) and
+    an elementwise sigmoid gate."""
+
+    heads: int
+    dim: int
+    vdim: int
+    decay: Tuple[float, ...]
+
+
+@dataclass(frozen=True)
+class SSDMixerSpec:
+    """Mamba-2 state-space layer: one projection gives gate z, input x, the
+    grouped B and C and a step per head; x|B|C pass a short causal filter with
+    bias and silu; per head S_t = exp(-exp(A_log) dt) S_(t-1) + dt B_t x_t^T
+    ([state, vdim]), y_t = S_t^T C_t + D x_t; y * silu(z) is RMS-normed in
+    `norm_groups` equal parts."""
+
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int = 1
+
+
 MixerSpec = Union[AttnMixerSpec, DeltaMixerSpec, ParallelMixerSpec,
-                  TiedAttnMixerSpec, LatentAttnMixerSpec, MLSTMMixerSpec]
+                  TiedAttnMixerSpec, LatentAttnMixerSpec, MLSTMMixerSpec,
+                  DecayAttnMixerSpec, SSDMixerSpec]
 
 
 @dataclass(frozen=True)
@@ -134,7 +178,20 @@ class RoutedExpertsSpec:
     ``groups`` / ``keep``: the experts form `groups` equal runs of neighbours;
     a run is worth the sum of its `group_rank` largest scores and only experts
     of the `keep` best runs can be chosen (groups = keep = 1: no restriction).
-    ``act``: "relu2" = the square of relu between the two matrices."""
+    ``act``: "relu2" = the square of relu between the two matrices.
+
+    ``router`` "softmax": scores are the softmax over all router outputs;
+    the choice (and the worth of a group, with `group_rank` 1 its largest
+    member) looks at score + `correction` (a learned vector), experts outside
+    the kept groups cannot be chosen whatever their sign, and the weights are
+    the plain scores times `route_scale`, not renormalised. The last
+    `identity` router outputs are identity experts (result = the input) that
+    have no matrices; they belong to the groups like the others.
+    ``act`` "clamped_glu": three-matrix experts, g = min(gate h, limit),
+    u = clamp(up h, -limit, limit), down(g sigmoid(1.702 g) (u + 1)).
+    ``shared_ff``: inner width of a shared expert of the same form (own
+    `shared_limit`) that every token uses, weighted by the sigmoid of a
+    one-row projection of the input; 0 = none."""
 
     ff: int
     experts: int
@@ -144,6 +201,12 @@ class RoutedExpertsSpec:
     group_rank: int = 2
     router: str = "sigmoid"
     act: str = "relu2"
+    identity: int = 0
+    route_scale: float = 1.0
+    correction: bool = False
+    limit: float = 0.0
+    shared_ff: int = 0
+    shared_limit: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -209,6 +272,8 @@ class HybridSpec:
             return self._sandwich_param_count()
         if self.arch == "vukotar":
             return self._parallel_param_count(active=False)
+        if self.arch == "nosalorn":
+            return self._prenorm_param_count(active=False)
         for layer in self.layers:
             m = layer.mixer
             if isinstance(m, ParallelMixerSpec):
@@ -266,9 +331,41 @@ class HybridSpec:
                 n += (e.top if active else e.experts) * 2 * h * e.ff
         return n
 
+    def _prenorm_param_count(self, active: bool) -> int:
+        """Pre-norm layers with attention / decay attention / state-space
+        mixers and SwiGLU or routed clamped-GLU feed-forwards."""
+        h = self.hidden_size
+        n = 2 * self.vocab_size * h + h
+        for layer in self.layers:
+            m = layer.mixer
+            n += h
+            if isinstance(m, AttnMixerSpec):
+                cols = m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)
+                n += (h + 1) * cols + m.heads * m.vdim * h + int(m.v_mix)
+            elif isinstance(m, DecayAttnMixerSpec):
+                hv = m.heads * m.vdim
+                n += h * (2 * m.heads * m.dim + 2 * hv) + hv + hv * h
+            elif isinstance(m, SSDMixerSpec):
+                inner, bc = m.heads * m.vdim, 2 * m.groups * m.state
+                n += h * (2 * inner + bc + m.heads)
+                n += (inner + bc) * (m.conv + 1) + 3 * m.heads + inner
+                n += inner * h
+            if layer.ff:
+                n += h + 3 * h * layer.ff
+            if layer.moe:
+                e = layer.moe
+                n += h + (e.experts + e.identity) * (h + 1)
+                n += (min(e.top, e.experts) if active else e.experts) \
+                    * 3 * h * e.ff
+                if e.shared_ff:
+                    n += 3 * h * e.shared_ff + h
+        return n
+
     def active_param_count(self) -> int:
         if self.arch == "vukotar":
             return self._parallel_param_count(active=True)
+        if self.arch == "nosalorn":
+            return self._prenorm_param_count(active=True)
         return self.param_count()
 
 
@@ -472,3 +569,102 @@ def vukotar_spec(config: dict, name: str = "vukotar",
         logit_softcap=float(config.get("logit_softcap", 0.0) or 0.0),
         tie_embeddings=True,
         num_experts=max((l.moe.experts if l.moe else 0) for l in layers))
+
+
+def nosalorn_spec(config: dict, name: str = "nosalorn",
+                  checkpoint_dir: Optional[str] = None,
+                  tensor_shapes: Optional[dict] = None) -> HybridSpec:
+    """Build the spec of a Nosalorn checkpoint from its ``config.json``: a
+    list of pre-norm layers (weighted RMS norms), each with a windowed
+    rotary attention (biased projections, YaRN frequencies, kept first
+    tokens, values blended with the first blending layer's), a fixed-decay
+    linear attention or a Mamba-2 mixer, and an optional SwiGLU or
+    routed-experts feed-forward; scaled token embedding, untied head, scaled
+    logits."""
+    layers = []
+    first_mix = None
+    for i, lc in enumerate(config["layers"]):
+        kind = lc["type"]
+        m = lc["mixer"]
+        if kind == "attention":
+            rot = m.get("rot") or {}
+            mask = m.get("mask") or {}
+            sc = rot.get("scaling")
+            mixer: MixerSpec = AttnMixerSpec(
+                heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+                dim=int(m["dim"]), vdim=int(m["vdim"]),
+                scale=float(m["scale"]), rot_dims=int(rot.get("dims", 0)),
+                rot_base=float(rot.get("base", 10000.0)),
+                window=int(mask.get("size", 0) or 0),
+                keep_first=int(mask.get("keep_first", 0) or 0),
+                rot_scaling=(float(sc["factor"]), float(sc["original"]),
+                             float(sc["fast"]), float(sc["slow"]))
+                if sc else None,
+                qk_norm=False, bias=True, out_bias=False, out_gate=False,
+                v_mix=bool(m.get("v_mix", False)))
+            if mixer.v_mix:
+                cols = mixer.kv_heads * mixer.vdim
+                if first_mix is None:
+                    first_mix = cols
+                elif cols != first_mix:
+                    raise ValueError(
+                        f"layer {i}: blended values must be as wide as the "
+                        f"first blending layer's ({first_mix})")
+        elif kind == "lightning":
+            mixer = DecayAttnMixerSpec(
+                heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                decay=tuple(float(d) for d in m["decay"]))
+            if len(mixer.decay) != mixer.heads:
+                raise ValueError(f"layer {i}: one decay per head is needed")
+        elif kind == "mamba2":
+            mixer = SSDMixerSpec(
+                heads=int(m["heads"]), vdim=int(m["vdim"]),
+                state=int(m["state"]), groups=int(m.get("groups", 1)),
+                conv=int(m["conv"]), norm_groups=int(m.get("norm_groups", 1)))
+            if mixer.heads % mixer.groups or \
+                    (mixer.heads * mixer.vdim) % mixer.norm_groups:
+                raise ValueError(f"layer {i}: heads must split into the "
+                                 f"groups and the width into the norm groups")
+        else:
+            raise ValueError(f"unknown layer type {kind!r} in layer {i}")
+        mlp = lc.get("mlp")
+        ff, moe = 0, None
+        if mlp is not None:
+            fk = mlp.get("kind", "dense")
+            if fk == "dense":
+                ff = int(mlp["ff"])
+            elif fk == "moe":
+                r = mlp["router"]
+                g = r.get("groups") or {"count": 1, "keep": 1}
+                sh = mlp.get("shared") or {}
+                moe = RoutedExpertsSpec(
+                    ff=int(mlp["expert"]["ff"]), experts=int(r["experts"]),
+                    top=int(r["top"]), groups=int(g["count"]),
+                    keep=int(g["keep"]), group_rank=1, router="softmax",
+                    act="clamped_glu", identity=int(r.get("identity", 0) or 0),
+                    route_scale=float(r.get("scale", 1.0)), correction=True,
+                    limit=float(mlp["expert"]["limit"]),
+                    shared_ff=int(sh.get("ff", 0) or 0),
+                    shared_limit=float(sh.get("limit", 0.0) or 0.0))
+                n = moe.experts + moe.identity
+                if n % moe.groups or not 1 <= moe.keep <= moe.groups:
+                    raise ValueError(
+                        f"layer {i}: experts and identity experts must split "
+                        f"into equal groups, of which 1..groups are kept")
+                if moe.top > moe.keep * (n // moe.groups):
+                    raise ValueError(f"layer {i}: the kept groups hold fewer "
+                                     f"experts than a token uses")
+            else:
+                raise ValueError(f"unknown feed-forward kind {fk!r}")
+        layers.append(HybridLayerSpec(kind=kind, mixer=mixer, ff=ff,
+                                      ff_kind="swiglu", moe=moe))
+    return HybridSpec(
+        name=name, arch="nosalorn", hidden_size=int(config["width"]),
+        vocab_size=int(config["vocab"]), layers=tuple(layers),
+        norm_eps=float(config["norm"]["eps"]),
+        max_context=int(config.get("max_context", 1 << 20)),
+        checkpoint_dir=checkpoint_dir,
+        embed_scale=float((config.get("embedding") or {}).get("scale", 1.0)),
+        logit_scale=float(config.get("logit_scale", 1.0)),
+        num_experts=max([(l.moe.experts if l.moe else 0) for l in layers]
+                        + [0]))

@@ -180,7 +180,7 @@ def safetensors_shapes(path: str) -> Dict[str, tuple]:
 def spec_from_dir(path: str, name: Optional[str] = None):
     """Spec of a checkpoint directory, chosen by its ``config.json``.
 
-    ``"architecture": "Vodinex"``, ``"Ruludra"`` or ``"Vukotar"`` gives a layer-list
+    ``"architecture": "Vodinex"``, ``"Ruludra"``, ``"Vukotar"`` or ``"Nosalorn"`` gives a layer-list
     :class:`HybridSpec`;
     a Hugging-Face style ``"architectures": ["Qwen3...ForCausalLM"]`` gives a
     :class:`ModelSpec` of the Qwen3 family. The returned spec remembers the
@@ -209,6 +209,11 @@ def spec_from_dir(path: str, name: Optional[str] = None):
 
         return vukotar_spec(cfg, name=name, checkpoint_dir=path,
                             tensor_shapes=safetensors_shapes(path))
+    if arch == "Nosalorn":
+        from .hybrid_spec import nosalorn_spec
+
+        return nosalorn_spec(cfg, name=name, checkpoint_dir=path,
+                             tensor_shapes=safetensors_shapes(path))
     if arch and arch.startswith("Qwen3"):
         moe = int(cfg.get("num_experts", 0) or 0)
         heads = int(cfg["num_attention_heads"])
@@ -254,6 +259,10 @@ def build_model(spec, dtype, max_len: int, tp=None, moe_ep: bool = False):
         from .vukotar import VukotarModel
 
         return VukotarModel(spec, dtype, max_len, tp)
+    if spec.arch == "nosalorn":
+        from .nosalorn import NosalornModel
+
+        return NosalornModel(spec, dtype, max_len, tp)
     from .qwen3 import Qwen3Model
 
     return Qwen3Model(spec, dtype, max_len, tp, moe_ep=moe_ep)

@@ -113,7 +113,7 @@ class ParallelBlock(nn.Module):
                    cache_idx=cache_idx)
         y = self.out_proj(mix_in)
         if self.experts is not None:
-            rows, padpos, wts = self.experts(h)
+            rows, padpos, wts, _ = self.experts(h)
             hops.dyt_residual(x, y, self.ls1, None, self.ls2, rows, padpos,
                               wts, norm=next_norm, h_out=h)
         else:

@@ -221,15 +221,24 @@ def rope_inv_freq(rot_dims: int, base: float) -> torch.Tensor:
 
 
 def attn_prep(proj, q_off, k_off, v_off, H, G, dk, dv, q_norm_w, k_norm_w,
-              eps, inv_freq, positions, slot_mapping, k_cache, v_cache):
+              eps, inv_freq, positions, slot_mapping, k_cache, v_cache,
+              rot_amp: float = 1.0, v_first=None, v_first_off: int = 0,
+              v_lambda=None):
     """Split q/k/v sections out of `proj`, per-head RMS norm on q and k
     (weights may be None), rotate the first 2*len(inv_freq) dims of each q/k
-    head (rotate-half pairing, fp32 angles = position * inv_freq), write k and
-    v into their paged caches and return q [T, H, dk]."""
+    head (rotate-half pairing, fp32 angles = position * inv_freq, cos and sin
+    times `rot_amp`), write k and v into their paged caches and return q
+    [T, H, dk]. With `v_first` (a buffer whose columns v_first_off.. hold
+    another layer's values of the same tokens) and `v_lambda` (0-d fp32) the
+    cached values are (1 - lambda) v + lambda v_first."""
     T = proj.shape[0]
     q = proj[:, q_off:q_off + H * dk].float().reshape(T, H, dk)
     k = proj[:, k_off:k_off + G * dk].float().reshape(T, G, dk)
     v = proj[:, v_off:v_off + G * dv].reshape(T, G, dv)
+    if v_first is not None:
+        lam = v_lambda.float()
+        v = ((1.0 - lam) * v.float() + lam * v_first[
+            :, v_first_off:v_first_off + G * dv].float().reshape(T, G, dv))
 
     def norm(x, w):
         if w is None:
@@ -241,6 +250,8 @@ def attn_prep(proj, q_off, k_off, v_off, H, G, dk, dv, q_norm_w, k_norm_w,
     if half:
         ang = positions.to(torch.float32).unsqueeze(1) * inv_freq.float().unsqueeze(0)
         c, s = ang.cos().unsqueeze(1), ang.sin().unsqueeze(1)
+        if rot_amp != 1.0:
+            c, s = c * rot_amp, s * rot_amp
 
         def rot(x):
             a, b, rest = x[..., :half], x[..., half:2 * half], x[..., 2 * half:]
@@ -258,10 +269,11 @@ def attn_prep(proj, q_off, k_off, v_off, H, G, dk, dv, q_norm_w, k_norm_w,
 def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
                     query_start_locs, scale, chunk, window, proj, gate_off,
                     out, out_off, out_scale, bias_r1=None, bias_r2=None,
-                    sink=False):
+                    sink=False, keep_first: int = 0):
     """Softmax attention of each sequence's new tokens over its cached keys
     under a local mask: query at position i sees j <= i with
-    j >= (i // chunk) * chunk (chunk > 0) and j > i - window (window > 0).
+    j >= (i // chunk) * chunk (chunk > 0) and j > i - window (window > 0);
+    keys j < keep_first stay visible whatever the window says.
     Head h's result is multiplied by out_scale * sigmoid(proj[t, gate_off+h])
     (gate_off < 0: no gate) and written to out[t, out_off + h*dv : ...].
     With bias_r1 / bias_r2 (fp32 [H]) the score of query i and key j is
@@ -295,7 +307,7 @@ def local_attention(q, k_cache, v_cache, block_tables, seq_lens,
         if chunk > 0:
             hidden = hidden | (kpos < (qpos // chunk) * chunk)
         if window > 0:
-            hidden = hidden | (kpos <= qpos - window)
+            hidden = hidden | ((kpos <= qpos - window) & (kpos >= keep_first))
         scores.masked_fill_(hidden.unsqueeze(0), float("-inf"))
         if sink:
             zero = torch.zeros(H, nq, 1, dtype=scores.dtype, device=q.device)
@@ -665,3 +677,252 @@ def moe_dispatch(idx, experts: int, bm: int):
 def softcap(logits, cap: float):
     """cap * tanh(logits / cap) in fp32."""
     return cap * torch.tanh(logits.float() / cap)
+
+
+# --------------------------------------------------------------------------
+# Pre-norm layers with a fused residual + routed-experts gather, YaRN
+# frequencies, gated linear units, a softmax router with identity experts,
+# and decay recurrences (fixed-decay linear attention, Mamba-2).
+# --------------------------------------------------------------------------
+
+GLU_GELU_TANH, GLU_SILU, GLU_CLAMPED = 0, 1, 2
+
+
+def yarn_inv_freq(rot_dims: int, base: float, scaling=None):
+    """(fp32 [rot_dims/2] frequencies, amplitude of cos / sin). `scaling` =
+    (factor, original length, fast turns, slow turns): with
+    d(t) = rot_dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(
+    d(fast)), 0), hi = min(ceil(d(slow)), rot_dims - 1) and ramp_i =
+    clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns at
+    f_i / factor * ramp_i + f_i (1 - ramp_i); amplitude 0.1 ln(factor) + 1.
+    Computed in fp64 and rounded once."""
+    import math
+
+    half = rot_dims // 2
+    i = torch.arange(half, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / max(1, rot_dims))
+    if not scaling:
+        return f.float(), 1.0
+    factor, orig, fast, slow = (float(z) for z in scaling)
+
+    def d(turns: float) -> float:
+        return rot_dims * math.log(orig / (2.0 * math.pi * turns)) / (
+            2.0 * math.log(float(base)))
+
+    lo = max(math.floor(d(fast)), 0)
+    hi = min(math.ceil(d(slow)), rot_dims - 1)
+    ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    f = f / factor * ramp + f * (1.0 - ramp)
+    return f.float(), 0.1 * math.log(factor) + 1.0
+
+
+def glu_mul(proj, gate_off: int, up_off: int, ff: int, act: int,
+            limit: float = 0.0):
+    """act(gate) * up over two sections of `proj`: GLU_GELU_TANH, GLU_SILU,
+    or GLU_CLAMPED: g = min(gate, limit), u = clamp(up, -limit, limit),
+    g sigmoid(1.702 g) (u + 1)."""
+    g = proj[:, gate_off:gate_off + ff].float()
+    u = proj[:, up_off:up_off + ff].float()
+    if act == GLU_GELU_TANH:
+        y = gelu_tanh(g) * u
+    elif act == GLU_SILU:
+        y = g * torch.sigmoid(g) * u
+    else:
+        g = g.clamp(max=limit)
+        y = g * torch.sigmoid(1.702 * g) * (u.clamp(-limit, limit) + 1.0)
+    return y.to(proj.dtype)
+
+
+def add_rmsnorm(x, y, rows, padpos, wts, idw, h_in, y2, proj2, sg_off,
+                norm_w, eps: float, h_out):
+    """x (fp32 [T, W], in place) += y (optional) + sum_j wts[t, j] *
+    rows[padpos[t, j]] over the pairs with wts != 0 (optional) + idw[t] *
+    h_in[t] (optional) + sigmoid(proj2[t, sg_off]) * y2[t] (optional; sg_off
+    < 0: no gate). Then h_out = x / sqrt(mean(x^2) + eps) * norm_w, unless
+    h_out is None."""
+    add = None
+
+    def acc(a, b):
+        return b if a is None else a + b
+
+    if y is not None:
+        add = acc(add, y.float())
+    if rows is not None:
+        live = (wts != 0).unsqueeze(-1)
+        r = torch.where(live, rows[padpos.long().clamp(min=0)].float(),
+                        torch.zeros((), dtype=torch.float32, device=x.device))
+        add = acc(add, (r * wts.unsqueeze(-1)).sum(dim=1))
+    if idw is not None:
+        add = acc(add, idw.float().unsqueeze(-1) * h_in.float())
+    if y2 is not None:
+        z = y2.float()
+        if sg_off >= 0:
+            z = z * torch.sigmoid(proj2[:, sg_off:sg_off + 1].float())
+        add = acc(add, z)
+    if add is not None:
+        x.add_(add)
+    if h_out is not None:
+        h_out.copy_((x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+                     * norm_w.float()).to(h_out.dtype))
+
+
+def moe_route_softmax(logits, corr, top: int, groups: int, keep: int,
+                      n_real: int, scale: float):
+    """Softmax router over fp32 logits [T, n] (n = n_real experts + identity
+    experts). Choice scores are softmax + corr (corr may be None); the
+    outputs form `groups` equal runs of neighbours, a run is worth its
+    largest choice score, only members of the `keep` best runs can be chosen
+    (ties to the lower index), and the `top` largest choice scores among them
+    are. Returns (idx int32 [T, top], w fp32 [T, top], idw fp32 [T]): a chosen
+    expert has its softmax score times `scale` as weight; chosen identity
+    experts appear as index n_real with weight 0, and the sum of their
+    weights is idw."""
+    T, n = logits.shape
+    s = torch.softmax(logits.float(), dim=-1)
+    c = s if corr is None else s + corr.float()
+    if groups > 1:
+        size = n // groups
+        per = c.view(T, groups, size)
+        worth = per.max(dim=-1).values
+        order = torch.sort(worth, dim=-1, descending=True, stable=True).indices
+        allow = torch.zeros(T, groups, dtype=torch.bool, device=s.device)
+        allow.scatter_(1, order[:, :keep], True)
+        c = torch.where(allow.unsqueeze(-1), per,
+                        torch.full_like(per, float("-inf"))).reshape(T, n)
+    idx = torch.sort(c, dim=-1, descending=True, stable=True).indices[:, :top]
+    w = s.gather(1, idx) * scale
+    ident = idx >= n_real
+    idw = torch.where(ident, w, torch.zeros_like(w)).sum(-1)
+    w = torch.where(ident, torch.zeros_like(w), w)
+    idx = torch.where(ident, torch.full_like(idx, n_real), idx)
+    return idx.to(torch.int32), w, idw
+
+
+def glu_grouped_gemm(out, a, w, row_tok, tile_off, counts, bm: int,
+                     limit: float):
+    """Per-expert segments like `grouped_gemm`, gathered rows, w [E, 2*ff, K]
+    holding gate rows then up rows; out[r] = g sigmoid(1.702 g) (u + 1) with
+    g = min(gate, limit), u = clamp(up, -limit, limit)."""
+    E, N, K = w.shape
+    ff = N // 2
+    for e in range(E):
+        c = int(counts[e])
+        if c == 0:
+            continue
+        s0 = int(tile_off[e]) * bm
+        rows = a[row_tok[s0:s0 + c].long().clamp(min=0)].float()
+        g = (rows @ w[e, :ff].T.float()).clamp(max=limit)
+        u = (rows @ w[e, ff:].T.float()).clamp(-limit, limit)
+        out[s0:s0 + c] = (g * torch.sigmoid(1.702 * g) * (u + 1.0)).to(out.dtype)
+    return out
+
+
+def silu_sections(proj, offs, sizes):
+    """fp32 silu of column sections of `proj`: one [T, size] tensor each."""
+    outs = []
+    for o, n in zip(offs, sizes):
+        z = proj[:, o:o + n].float()
+        outs.append((z * torch.sigmoid(z)).contiguous())
+    return outs
+
+
+def ssd_prep(proj, xbc_off: int, dt_off: int, H: int, dv: int, G: int, N: int,
+             conv_w, conv_b, dt_bias, a_log, conv_state, state_slots,
+             query_start_locs, seq_lens):
+    """Inputs of the Mamba-2 recurrence for every new token. The x|B|C
+    section of `proj` (H*dv + 2*G*N channels) passes a causal depthwise
+    filter (`conv_w` [C, taps], last tap = current token, bias `conv_b`;
+    inputs before a sequence's start are zero; a continuing sequence's
+    history is conv_state[slot] = its last taps-1 raw inputs, time-major,
+    which is brought up to date) and silu. dt = softplus(dt section +
+    dt_bias), decay = exp(-exp(a_log) dt). Returns fp32 (x [T,H,dv],
+    B [T,G,N], C [T,G,N], decay [T,H], dt [T,H])."""
+    T = proj.shape[0]
+    inner = H * dv
+    Cn = inner + 2 * G * N
+    taps = conv_w.shape[1]
+    raw = proj[:, xbc_off:xbc_off + Cn].float()
+    y = torch.empty_like(raw)
+    wf = conv_w.float()
+    for s in range(seq_lens.numel()):
+        a, b = int(query_start_locs[s]), int(query_start_locs[s + 1])
+        n = b - a
+        if n == 0:
+            continue
+        start = int(seq_lens[s]) - n
+        slot = int(state_slots[s])
+        if taps > 1:
+            hist = (conv_state[slot].float() if start > 0
+                    else torch.zeros(taps - 1, Cn, dtype=torch.float32,
+                                     device=proj.device))
+            ext = torch.cat([hist, raw[a:b]], dim=0)
+            conv_state[slot] = ext[-(taps - 1):].to(conv_state.dtype)
+        else:
+            ext = raw[a:b]
+        acc = conv_b.float().unsqueeze(0).expand(n, Cn).clone()
+        for j in range(taps):
+            acc = acc + ext[j:j + n] * wf[:, j]
+        y[a:b] = acc * torch.sigmoid(acc)
+    x = y[:, :inner].reshape(T, H, dv).contiguous()
+    B = y[:, inner:inner + G * N].reshape(T, G, N).contiguous()
+    C = y[:, inner + G * N:].reshape(T, G, N).contiguous()
+    dt = torch.nn.functional.softplus(
+        proj[:, dt_off:dt_off + H].float() + dt_bias.float())
+    decay = torch.exp(-torch.exp(a_log.float()) * dt)
+    return x, B, C, decay.contiguous(), dt.contiguous()
+
+
+def decay_scan(q, k, v, decay, gain, skip, state, state_slots,
+               query_start_locs, seq_lens):
+    """Token-by-token decay recurrence per sequence and head, state[slot] =
+    S [H, dk, dv] (fp32, zero at a sequence's start):
+        S <- decay * S + gain * k v^T;   o = S^T q + skip * v.
+    q, k fp32 [T, G, dk] (head h reads group h // (H/G)); v fp32 [T, H, dv];
+    decay fp32 [T, H] or [H] (the same at every token); gain fp32 [T, H] or
+    None (1); skip fp32 [H] or None (0). Returns o [T, H, dv] fp32 and leaves
+    the new state in `state`."""
+    T, H, dv = v.shape
+    G = k.shape[1]
+    rep = H // G
+    o = torch.empty(T, H, dv, dtype=torch.float32, device=v.device)
+    for s in range(seq_lens.numel()):
+        a, b = int(query_start_locs[s]), int(query_start_locs[s + 1])
+        n = b - a
+        if n == 0:
+            continue
+        start = int(seq_lens[s]) - n
+        slot = int(state_slots[s])
+        St = (state[slot].clone() if start > 0
+              else torch.zeros_like(state[slot]))
+        for t in range(a, b):
+            kt = k[t].repeat_interleave(rep, dim=0)
+            qt = q[t].repeat_interleave(rep, dim=0)
+            d = decay if decay.dim() == 1 else decay[t]
+            kv = kt.unsqueeze(-1) * v[t].unsqueeze(1)
+            if gain is not None:
+                kv = kv * gain[t].view(H, 1, 1)
+            St = St * d.view(H, 1, 1) + kv
+            o[t] = torch.einsum("hkv,hk->hv", St, qt)
+            if skip is not None:
+                o[t] += skip.view(H, 1) * v[t]
+        state[slot] = St
+    return o
+
+
+def gated_group_norm(o, proj, g_off: int, norm_w, eps: float, groups: int,
+                     gate_first: bool, out, out_off: int):
+    """o fp32 [T, n] (any trailing shape), gate = the n columns of `proj` from
+    g_off. gate_first: y = o * silu(gate), then each of `groups` equal parts
+    of y divided by its root mean square, times norm_w. Otherwise: parts of o
+    normed, times norm_w, times sigmoid(gate). Written to
+    out[:, out_off : out_off + n]."""
+    T = o.shape[0]
+    y = o.reshape(T, -1)
+    n = y.shape[1]
+    g = proj[:, g_off:g_off + n].float()
+    if gate_first:
+        y = y * (g * torch.sigmoid(g))
+    y = _unit_rms(y.view(T, groups, n // groups), eps).reshape(T, n) * norm_w.float()
+    if not gate_first:
+        y = y * torch.sigmoid(g)
+    out[:, out_off:out_off + n] = y.to(out.dtype)
