@@ -79,7 +79,7 @@ def build_args():
                         "of 1b,8b,tiny); one JSON line per model")
     p.add_argument("--compare-models", type=str, default="vodinex,qwen3",
                    help="models of --arch-compare: comma list of vodinex, "
-                        "ruludra, vukotar, qwen3, qwen3moe (vukotar's "
+                        "ruludra, vukotar, nosalorn, qwen3, qwen3moe (vukotar's and nosalorn's "
                         "counterpart is qwen3moe)")
     p.add_argument("--compare-seqs", type=int, default=16)
     p.add_argument("--compare-prompt", type=int, default=2048)

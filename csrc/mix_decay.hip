@@ -58,6 +58,75 @@ __global__ void __launch_bounds__(256) ssd_prep_kernel(
   xbc[t * C + c] = acc * sigmoid_f(acc);
 }
 
+// bf16 fast path: a thread filters 8 consecutive channels of one token (one
+// 16-byte load a tap, two 16-byte stores); the steps and decays of a token are
+// made by the threads past the channel work. Needs C, the section start and
+// the row length to be multiples of 8.
+__global__ void __launch_bounds__(256) ssd_prep_vec_kernel(
+    float* __restrict__ xbc, float* __restrict__ decay, float* __restrict__ dt,
+    const u16* __restrict__ proj, long ld, int xbc_off, int dt_off,
+    const float* __restrict__ conv_wt, const float* __restrict__ conv_b,
+    int taps, const float* __restrict__ dt_bias,
+    const float* __restrict__ a_log, const float* __restrict__ conv_state,
+    const int* __restrict__ state_slots, const int* __restrict__ qlocs,
+    const int* __restrict__ seq_lens, const int* __restrict__ token_seq, long T,
+    int C, int H) {
+  const int C8 = C / 8;
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= T * C8) {
+    const long j = i - T * C8;
+    if (j >= T * H) return;
+    const long t = j / H;
+    const int h = (int)(j - t * H);
+    const float d = softplus_f(bf2f(proj[t * ld + dt_off + h]) + dt_bias[h]);
+    dt[j] = d;
+    decay[j] = expf(-expf(a_log[h]) * d);
+    return;
+  }
+  const long t = i / C8;
+  const int c = (int)(i - t * C8) * 8;
+  const int s = token_seq[t];
+  const int q0 = qlocs[s], n = qlocs[s + 1] - q0;
+  const int start = seq_lens[s] - n;
+  const int loc = (int)t - q0;
+  const float* hist = conv_state + (long)state_slots[s] * (taps - 1) * C + c;
+  float acc[8];
+  {
+    const f32x4 b0 = *(const f32x4*)(conv_b + c), b1 = *(const f32x4*)(conv_b + c + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { acc[e] = b0[e]; acc[e + 4] = b1[e]; }
+  }
+  for (int j = 0; j < taps; ++j) {
+    const int tau = loc - (taps - 1 - j);
+    float x[8];
+    if (tau >= 0) {
+      bf8_to_f32(*(const u16x8*)(proj + (long)(q0 + tau) * ld + xbc_off + c), x);
+    } else if (start > 0) {
+      const float* hr = hist + (long)(taps - 1 + tau) * C;
+      const f32x4 h0 = *(const f32x4*)hr, h1 = *(const f32x4*)(hr + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { x[e] = h0[e]; x[e + 4] = h1[e]; }
+    } else {
+      continue;
+    }
+    const float* wr = conv_wt + (long)j * C + c;
+    const f32x4 w0 = *(const f32x4*)wr, w1 = *(const f32x4*)(wr + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      acc[e] += w0[e] * x[e];
+      acc[e + 4] += w1[e] * x[e + 4];
+    }
+  }
+  f32x4 o0, o1;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    o0[e] = acc[e] * sigmoid_f(acc[e]);
+    o1[e] = acc[e + 4] * sigmoid_f(acc[e + 4]);
+  }
+  *(f32x4*)(xbc + t * C + c) = o0;
+  *(f32x4*)(xbc + t * C + c + 4) = o1;
+}
+
 // one thread per (sequence, channel): new history = last taps-1 raw inputs
 template <typename A>
 __global__ void __launch_bounds__(256) ssd_conv_update_kernel(
@@ -105,6 +174,13 @@ extern "C" void mix_ssd_prep(float* xbc, float* decay, float* dt,
                          0, s, conv_state, (const float*)proj, ld, xbc_off,
                          taps, state_slots, qlocs, seq_lens, S, C);
   } else {
+    if (C % 8 == 0 && xbc_off % 8 == 0 && ld % 8 == 0) {
+      const unsigned vgrid = (unsigned)((T * (C / 8) + T * H + 255) / 256);
+      hipLaunchKernelGGL(ssd_prep_vec_kernel, dim3(vgrid), dim3(256), 0, s, xbc,
+                         decay, dt, (const u16*)proj, ld, xbc_off, dt_off,
+                         conv_wt, conv_b, taps, dt_bias, a_log, conv_state,
+                         state_slots, qlocs, seq_lens, token_seq, T, C, H);
+    } else
     hipLaunchKernelGGL(ssd_prep_kernel<u16>, dim3(grid), dim3(256), 0, s, xbc,
                        decay, dt, (const u16*)proj, ld, xbc_off, dt_off,
                        conv_wt, conv_b, taps, dt_bias, a_log, conv_state,

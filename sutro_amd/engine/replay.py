@@ -69,6 +69,9 @@ def main(argv=None) -> int:
         enforce_eager=args.eager)
     eng = LLMEngine(cfg)
     os.makedirs(args.out, exist_ok=True)
+    sys.stdout.write(f"engine {spec.arch} on {device} in {args.dtype}, "
+                     f"{blocks} pages of {bs}\n")
+    sys.stdout.flush()
 
     live = {}
     for line in sys.stdin:

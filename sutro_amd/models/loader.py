@@ -62,12 +62,17 @@ def _load_by_targets(model: torch.nn.Module, path: str, strict: bool) -> int:
     """Models that publish `checkpoint_targets()` (checkpoint tensor name ->
     (parameter, dim, start, length, scale)) are filled section by section:
     the tensor, times `scale`, lands in parameter.narrow(dim, start, length);
-    dim None means a 0-d tensor. Every target must be met exactly once."""
+    dim None means a 0-d tensor. Every target must be met exactly once; a
+    name mapped to None is a tensor that may be present and is not used."""
     params: Dict[str, torch.nn.Parameter] = dict(model.named_parameters())
     targets = model.checkpoint_targets()
     seen = set()
     unexpected: List[str] = []
     for name, tensor in _iter_safetensors(path):
+        if name in targets and targets[name] is None:
+            # a tensor the model knows of but does not use: it may be there
+            seen.add(name)
+            continue
         tgt = targets.get(name)
         if tgt is None:
             unexpected.append(name)
@@ -96,7 +101,8 @@ def _load_by_targets(model: torch.nn.Module, path: str, strict: bool) -> int:
                         f"{pname}")
                 dst.copy_(src.to(p.dtype))
         seen.add(name)
-    missing = sorted(set(targets) - seen)
+    missing = sorted(k for k, v in targets.items()
+                     if v is not None and k not in seen)
     if strict and unexpected:
         raise ValueError(f"checkpoint has {len(unexpected)} tensors that map "
                          f"to no parameter: {unexpected[:6]}")

@@ -88,8 +88,10 @@ class PreNormBlock(nn.Module):
             prefix + "in_proj.", self.mixer.section_names("", ck)))
         if hasattr(self.mixer, "param_targets"):
             t.update(self.mixer.param_targets(prefix + "mixer.", ck))
-        if isinstance(self.mixer, LocalAttention) and self.mixer.spec.v_mix:
-            t[ck + ".vmix"] = (prefix + "mixer.v_lambda", None, 0, 0, 1.0)
+        if isinstance(self.mixer, LocalAttention):
+            # a layer that does not blend may still carry the (unused) weight
+            t[ck + ".vmix"] = (prefix + "mixer.v_lambda", None, 0, 0, 1.0) \
+                if self.mixer.spec.v_mix else None
         t[ck + ".o"] = (prefix + "out_proj.weight", 1, 0,
                         self.mixer.out_width, 1.0)
         if self.has_ff:

@@ -1,5 +1,5 @@
 """Prefill and decode throughput of the layer-list decoders (Vodinex,
-Ruludra, Vukotar) beside the Qwen3 decoder of equal size (same width, layers,
+Ruludra, Vukotar, Nosalorn) beside the Qwen3 decoder of equal size (same width, layers,
 heads, key/value heads, head size and feed-forward width; for Vukotar the
 Qwen3 mixture-of-experts decoder with as many experts of the same inner
 width and as many choices a token), all with random weights, all through the
@@ -20,8 +20,9 @@ import torch
 
 from ..engine.config import EngineConfig
 from ..engine.engine import LLMEngine
-from ..models.hybrid_spec import (AttnMixerSpec, DeltaMixerSpec,
-                                  HybridLayerSpec, HybridSpec,
+from ..models.hybrid_spec import (AttnMixerSpec, DecayAttnMixerSpec,
+                                  DeltaMixerSpec, HybridLayerSpec, HybridSpec,
+                                  SSDMixerSpec,
                                   LatentAttnMixerSpec, MLSTMMixerSpec,
                                   ParallelMixerSpec, RoutedExpertsSpec,
                                   TiedAttnMixerSpec)
@@ -118,6 +119,47 @@ def parallel_spec(name: str) -> HybridSpec:
                       num_experts=MOE_EXPERTS)
 
 
+def prenorm_spec(name: str, window: int = 1024) -> HybridSpec:
+    """Nosalorn at the same width, depth, heads and head size: a Mamba-2
+    layer (state 128) with a dense SwiGLU feed-forward, then window-1024
+    rotary attention (64 kept first tokens, YaRN, blended values), fixed-decay
+    linear attention and attention again, each beside 28 clamped-GLU experts
+    + 4 identity experts (8 groups of 4, the best 4 stay, 4 a token, inner
+    width ff/4) and a gated shared expert of the same width."""
+    W, L, H, G, D, ff, V = SIZES[name]
+    attn = AttnMixerSpec(heads=H, kv_heads=G, dim=D, vdim=D, scale=D ** -0.5,
+                         rot_dims=D // 2, rot_base=10000.0, window=window,
+                         keep_first=64, rot_scaling=(4.0, 4096.0, 32.0, 1.0),
+                         qk_norm=False, bias=True, out_bias=False,
+                         out_gate=False, v_mix=True)
+    ssd = SSDMixerSpec(heads=H, vdim=D, state=min(128, D), groups=G, conv=4,
+                       norm_groups=G)
+    lin = DecayAttnMixerSpec(heads=H, dim=D, vdim=D, decay=tuple(
+        1.0 - 2.0 ** (-2.0 - 6.0 * i / max(1, H - 1)) for i in range(H)))
+    eff = max(64, ff // MOE_FF_DIV)
+    moe = RoutedExpertsSpec(ff=eff, experts=MOE_EXPERTS - 4, top=MOE_TOP,
+                            groups=8, keep=4, group_rank=1, router="softmax",
+                            act="clamped_glu", identity=4, route_scale=2.0,
+                            correction=True, limit=7.0, shared_ff=eff,
+                            shared_limit=7.0)
+    layers: List[HybridLayerSpec] = []
+    for i in range(L):
+        k = i % 4
+        if k == 0:
+            layers.append(HybridLayerSpec("mamba2", ssd, ff=ff,
+                                          ff_kind="swiglu"))
+        elif k == 2:
+            layers.append(HybridLayerSpec("lightning", lin, ff_kind="swiglu",
+                                          moe=moe))
+        else:
+            layers.append(HybridLayerSpec("attention", attn, ff_kind="swiglu",
+                                          moe=moe))
+    return HybridSpec(name=f"nosalorn-{name}", arch="nosalorn", hidden_size=W,
+                      vocab_size=V, layers=tuple(layers), norm_eps=1e-6,
+                      max_context=1 << 20, embed_scale=4.0, logit_scale=0.5,
+                      num_experts=MOE_EXPERTS - 4)
+
+
 def moe_spec(name: str) -> ModelSpec:
     """The Qwen3 mixture-of-experts decoder with as many experts of the same
     inner width and as many choices a token (softmax router, SwiGLU
@@ -190,7 +232,7 @@ def _measure(spec, device: str, seqs: int, prompt: int, steps: int,
 
 MAKERS = {"vodinex": hybrid_spec, "qwen3": dense_spec,
           "ruludra": sandwich_spec, "vukotar": parallel_spec,
-          "qwen3moe": moe_spec}
+          "qwen3moe": moe_spec, "nosalorn": prenorm_spec}
 
 
 def run_compare(sizes: List[str], device: str, seqs: int, prompt: int,
