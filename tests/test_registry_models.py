@@ -32,9 +32,11 @@ def test_model_generates(name):
 def test_registry_specs_are_coherent():
     """Structural sanity across ALL 40 servable specs: GQA divisibility, TP
     divisibility for the recommended degree, MoE fields paired."""
-    from sutro_amd.models.registry import MODEL_REGISTRY
+    from sutro_amd.models.registry import MODEL_REGISTRY, ModelSpec
 
     for name, s in MODEL_REGISTRY.items():
+        if not isinstance(s, ModelSpec):
+            continue    # a checkpoint directory another test registered
         assert s.num_heads % s.num_kv_heads == 0, name
         assert s.head_dim in (64, 128), name
         assert s.hidden_size % s.num_heads != -1  # defined
